@@ -1,0 +1,227 @@
+/*
+ * optimus_mi355x.h — C ABI of liboptimus_mi355x.so
+ *
+ * MI355X (gfx950) implementation of the single-GPU training hot path of
+ * IntelLabs/Optimus-LM: the fast MoE block's operators and the flat-buffer
+ * mixed-precision AdamW step.  These entry points are what a binding of the
+ * reference's native-op module (pybind module `pcl_xpu_customops`,
+ * pytorch_xpu_extensions/pcl.xpu.customops/csrc/ops/sparse_moe_block.sycl:538-548)
+ * and of its Python-level hot loops (optimus/models/common/moe.py,
+ * optimus/optimizers.py) would bind.
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer to contiguous row-major memory unless the
+ *     parameter is documented as "host";
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); every call
+ *     only enqueues work on it: no allocation, no host synchronisation;
+ *   - the caller allocates every output and zero-fills the buffers documented as
+ *     "pre-zeroed" (same ownership rule as the reference ops, moe.py:492-497, :336);
+ *   - return value: OM_OK or a negative OM_ERR_* code; nothing throws.
+ */
+#ifndef OPTIMUS_MI355X_H
+#define OPTIMUS_MI355X_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    OM_OK = 0,
+    OM_ERR_NULL = -1,      /* a required pointer is NULL                        */
+    OM_ERR_DTYPE = -2,     /* dtype code not supported by this entry point      */
+    OM_ERR_SHAPE = -3,     /* sizes violate a documented constraint             */
+    OM_ERR_ALIGN = -4,     /* pointer / row pitch not aligned as documented     */
+    OM_ERR_LAUNCH = -5,    /* the HIP runtime rejected a launch                 */
+    OM_ERR_WORKSPACE = -6  /* workspace too small                               */
+};
+
+/* element types */
+enum { OM_F32 = 0, OM_BF16 = 1 };
+/* index types of `selected_experts` (the reference dispatches kLong, else int32) */
+enum { OM_I32 = 0, OM_I64 = 1 };
+
+/* Library version and the GPU architecture the kernels were compiled for ("gfx950"). */
+int om_version(void);
+const char *om_arch(void);
+const char *om_strerror(int code);
+
+/* ------------------------------------------------------------------------------------
+ * Flat-buffer mixed-precision AdamW step
+ * replaces: the chunked 13-op elementwise sequence of MixedPrecisionAdamW.step,
+ *           optimus/optimizers.py:162-205 (formula restated at optimizers.py:1745-1760).
+ * One pass over n elements:  g=float(grad); m=m*b1+(1-b1)*g; v=v*b2+(1-b2)*g*g;
+ *   w += -lr*(m/(1-b1^t))/(sqrt(v/(1-b2^t))+eps); if wd>0: w += (-lr*wd)*w; param=cast(w).
+ * param_dtype OM_BF16: param, grad are bf16; master/exp_avg/exp_avg_sq fp32.
+ * param_dtype OM_F32 : grad fp32 and `master` IS the parameter buffer; `param` is ignored
+ *                      (the reference aliases them, optimizers.py:100-102).
+ * `step` is t = step_id + 1 (1-based).  All five buffers must be 16-byte aligned.
+ * n may exceed 2^31.                                                                    */
+int om_adamw_step(void *param, const void *grad, float *master, float *exp_avg,
+                  float *exp_avg_sq, int64_t n, double lr, double beta1, double beta2,
+                  double eps, double weight_decay, int64_t step, int param_dtype,
+                  void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Routers
+ * om_route_softmax_topk replaces optimus/models/common/moe.py:467-471
+ *   (= optimus/models/olmoe/modeling_olmoe.py:295-299): fp32 softmax over N experts,
+ *   top-K by (probability desc, expert index asc), optional renormalisation, cast.
+ *   logits [T,N] (OM_F32 or OM_BF16); weights_out [T,K] (weights_dtype);
+ *   experts_out [T,K] int64, in descending-probability order.  N <= 512, K <= min(N,64).
+ * om_route_softmax_topk_bwd is the backward of the same expression (autograd in the
+ *   reference): dlogits [T,N] in logits dtype from dweights [T,K].                      */
+int om_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int N, int K,
+                          int norm_topk_prob, void *weights_out, int weights_dtype,
+                          int64_t *experts_out, void *stream);
+int om_route_softmax_topk_bwd(const void *logits, int logits_dtype, const int64_t *experts,
+                              const void *dweights, int weights_dtype, int64_t T, int N, int K,
+                              int norm_topk_prob, void *dlogits, void *stream);
+
+/* om_route_sigmoid_group_topk replaces DeepseekV3ParallelTopkRouter.get_topk_indices and
+ *   the weight computation of its forward,
+ *   optimus/models/deepseek_v3/modeling_deepseek_v3.py:164-180 and :185-191:
+ *   scores = sigmoid(logits); choice = scores + bias; group score = sum of the top-2 choice
+ *   values of each of n_group contiguous groups; the topk_group best groups keep their
+ *   choice values, all others become 0.0; experts = top-K of that; weights = scores at the
+ *   experts, divided by (sum + 1e-20) when norm_topk_prob, times routed_scaling_factor.
+ *   logits [T,N] fp32, bias [N] fp32 -> experts_out [T,K] int64 (descending choice value,
+ *   lower index first among equals), weights_out [T,K] fp32.  N <= 512, N % n_group == 0.
+ * om_route_sigmoid_topk_bwd: dlogits [T,N] fp32 (dense, zero off the selected experts).   */
+int om_route_sigmoid_group_topk(const float *logits, const float *bias, int64_t T, int N,
+                                int n_group, int topk_group, int K, int norm_topk_prob,
+                                double routed_scaling_factor, int64_t *experts_out,
+                                float *weights_out, void *stream);
+int om_route_sigmoid_topk_bwd(const float *logits, const int64_t *experts, const float *dweights,
+                              int64_t T, int N, int K, int norm_topk_prob,
+                              double routed_scaling_factor, float *dlogits, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Token permutation (index construction)
+ * om_moe_sort fuses the reference's K1 + K2 + K3:
+ *   compute_partial_token_counts      sparse_moe_block.sycl:108-173
+ *   the two cumsums and the host read moe.py:513-520
+ *   compute_input_and_output_indices  sparse_moe_block.sycl:175-280
+ * into a stable counting sort of the (token, k) pairs whose expert lies in
+ * [expert_start_idx, expert_end_idx).  Results are identical to the reference's:
+ *   cum_token_counts [NR+1], cum_expert_counts_ep [T+1], and — for the TR =
+ *   cum_token_counts[NR] routed rows — input_indices, output_indices,
+ *   selected_experts_indices (each with room for T*K entries; entries >= TR untouched).
+ * All outputs stay on the device; nothing is read back.
+ * workspace: om_moe_sort_workspace_bytes(T, K, NR) bytes, 4-byte aligned, no pre-zeroing. */
+int64_t om_moe_sort_workspace_bytes(int64_t T, int K, int NR);
+int om_moe_sort(const void *selected_experts, int index_dtype, int64_t T, int K,
+                int expert_start_idx, int expert_end_idx, int32_t *cum_token_counts,
+                int32_t *cum_expert_counts_ep, int32_t *input_indices, int32_t *output_indices,
+                int32_t *selected_experts_indices, void *workspace, int64_t workspace_bytes,
+                void *stream);
+
+/* The reference's two index kernels with their own table layout, for callers of the
+ * pybind module that still run K2 (torch.cumsum) themselves.
+ * replaces: compute_partial_token_counts      sparse_moe_block.sycl:138-173
+ *           compute_input_and_output_indices  sparse_moe_block.sycl:217-280
+ * partial_token_counts [NR,TH] and input_increment_buffer [NR,TH] are pre-zeroed by the
+ * caller and updated in place; TB = T / TH tokens per table column (T % TH == 0).        */
+int om_compute_partial_token_counts(const void *selected_experts, int index_dtype,
+                                    int32_t *partial_token_counts, int32_t *expert_counts_ep,
+                                    int expert_start_idx, int expert_end_idx, int64_t T, int K,
+                                    int64_t TH, void *stream);
+int om_compute_input_and_output_indices(const void *selected_experts, int index_dtype,
+                                        const int32_t *partial_cum_token_counts,
+                                        int32_t *input_increment_buffer,
+                                        const int32_t *cum_expert_counts_ep,
+                                        int32_t *selected_experts_indices, int32_t *input_indices,
+                                        int32_t *output_indices, int expert_start_idx,
+                                        int expert_end_idx, int64_t T, int K, int64_t TH,
+                                        void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Row movers (dtype OM_F32 or OM_BF16 for the activations; fp32 accumulation, one rounding)
+ * om_index_add                    replaces index_add_op      sparse_moe_block.sycl:24-54
+ *     output[indices[c],:] += input[c,:]   (atomic per element: duplicates are summed)
+ * om_index_gather                 replaces index_gather      sparse_moe_block.sycl:75-106
+ *     output[o,:] = input[indices[o],:]
+ * om_shuffle_sub_matrix_reduce    replaces shuffle_sub_matrix_reduce   .sycl:505-532
+ *     hidden_grad[t,:] = sum_{i in [cum_ep[t],cum_ep[t+1])} ggemm_input_grad[output_indices[i],:]
+ * om_reduce_ggemm_output          replaces reduce_ggemm_output         .sycl:314-362
+ *     final[t,:] = sum_i w[t, sel_idx[i]] * ggemm_output[output_indices[i],:]
+ *     (weights_dtype may be OM_F32 while dtype is OM_BF16: the DeepSeek-V3 block keeps its
+ *      routing weights in fp32, modeling_deepseek_v3.py:222-239)
+ * om_reduce_ggemm_output_backward replaces reduce_ggemm_output_backward .sycl:425-475
+ *     dy[pos,:] = w[t,k] * dout[t,:];  dw[t,k] = <y[pos,:], dout[t,:]>;  dw pre-zeroed.      */
+int om_index_add(const void *input, void *output, const int32_t *indices, int64_t C, int64_t E,
+                 int dtype, void *stream);
+int om_index_gather(const void *input, const int32_t *indices, void *output, int64_t O,
+                    int64_t E, int dtype, void *stream);
+int om_shuffle_sub_matrix_reduce(const void *ggemm_input_grad, const int32_t *cum_expert_counts_ep,
+                                 const int32_t *output_indices, void *hidden_states_grad,
+                                 int64_t T, int64_t E, int dtype, void *stream);
+int om_reduce_ggemm_output(const void *ggemm_output, const void *routing_weights,
+                           const int32_t *cum_expert_counts_ep,
+                           const int32_t *selected_experts_indices, const int32_t *output_indices,
+                           void *final_hidden_states, int64_t T, int K, int64_t E, int dtype,
+                           int weights_dtype, int skip_weights_scaling, void *stream);
+int om_reduce_ggemm_output_backward(const void *final_hidden_states_grad, const void *ggemm_output,
+                                    const void *routing_weights,
+                                    const int32_t *selected_experts_indices,
+                                    const int32_t *input_indices, const int32_t *output_indices,
+                                    void *ggemm_output_grad, void *routing_weights_grad,
+                                    int64_t RT, int K, int64_t E, int dtype, int weights_dtype,
+                                    void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Grouped expert GEMMs (bf16 operands, fp32 MFMA accumulation, bf16 results)
+ * The G experts own the row segments [cum_token_counts[g], cum_token_counts[g+1]) of the
+ * activation matrices; cum_token_counts [G+1] is a DEVICE int32 array (no host copy, no
+ * max_tokens_per_expert: the kernels size their work from `rows`, an upper bound on
+ * cum_token_counts[G] known to the host, e.g. the allocated row count).
+ * replaces GroupedGemmFunction, optimus/models/common/moe.py:163-215, whose tiling
+ * specification is optimus/kernels/merged_mlp_triton_kernels.py:8-269:
+ *   om_grouped_gemm_fwd    out[s:e,:]  = in[s:e,:]   @ W[g].T      (W [G,N,K] "out,in")
+ *   om_grouped_gemm_dgrad  din[s:e,:]  = dout[s:e,:] @ W[g]
+ *   om_grouped_gemm_wgrad  dW[g]       = dout[s:e,:].T @ in[s:e,:]  (zeros when s == e)
+ * w_stride: elements between the matrices of consecutive experts in `weight` /
+ * `weight_grad`; 0 means densely packed (N*K, the merged [G,N,K] layout).  A larger stride
+ * serves per-expert nn.Linear weights that sit at a constant pitch inside one flat buffer.
+ * N and K must be multiples of 128.                                                       */
+int om_grouped_gemm_fwd(const void *input, const void *weight, void *output,
+                        const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                        int64_t w_stride, void *stream);
+int om_grouped_gemm_dgrad(const void *output_grad, const void *weight, void *input_grad,
+                          const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                          int64_t w_stride, void *stream);
+int om_grouped_gemm_wgrad(const void *output_grad, const void *input, void *weight_grad,
+                          const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                          int64_t w_stride, void *stream);
+
+/* Merged-MLP fusions, replacing the three GroupedGemmFunction calls and the two torch
+ * elementwise ops of MergedMLP.forward (moe.py:396-405) and their autograd backward:
+ *   om_merged_mlp_gate_up_fwd : g = x@Wg[e].T, u = x@Wu[e].T, h = silu(g)*u in one kernel
+ *                               (x [rows,H]; Wg,Wu [G,I,H]; g,u,h [rows,I])
+ *   om_merged_mlp_down_dgrad  : dh = dy@Wd[e] fused with the SwiGLU backward
+ *                               du = dh*silu(g), dg = dh*u*sig(g)*(1+g*(1-sig(g)))
+ *                               (dy [rows,H]; Wd [G,H,I]; g,u in; dg,du out [rows,I])
+ *   om_merged_mlp_gate_up_dgrad: dx = dg@Wg[e] + du@Wu[e] with one accumulator.
+ * Weight gradients use om_grouped_gemm_wgrad.                                             */
+int om_merged_mlp_gate_up_fwd(const void *x, const void *w_gate, const void *w_up, void *g,
+                              void *u, void *h, const int32_t *cum_token_counts, int64_t rows,
+                              int G, int I, int H, int64_t w_stride, void *stream);
+int om_merged_mlp_down_dgrad(const void *dy, const void *w_down, const void *g, const void *u,
+                             void *dg, void *du, const int32_t *cum_token_counts, int64_t rows,
+                             int G, int I, int H, int64_t w_stride, void *stream);
+int om_merged_mlp_gate_up_dgrad(const void *dg, const void *du, const void *w_gate,
+                                const void *w_up, void *dx, const int32_t *cum_token_counts,
+                                int64_t rows, int G, int I, int H, int64_t w_stride,
+                                void *stream);
+
+/* Stand-alone SwiGLU glue (moe.py:401-402 forward; moe.py:37-41 and :133-147 backward),
+ * for callers that keep the three GEMMs separate.  n elements, dtype OM_F32 or OM_BF16.   */
+int om_swiglu_fwd(const void *g, const void *u, void *h, int64_t n, int dtype, void *stream);
+int om_swiglu_bwd(const void *dh, const void *g, const void *u, void *dg, void *du, int64_t n,
+                  int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OPTIMUS_MI355X_H */

@@ -1,0 +1,199 @@
+// Flat-buffer mixed-precision AdamW: one coalesced, vectorised pass (HBM-bound).
+// Algorithmic traffic per element: read grad 2 + master 4 + m 4 + v 4, write master 4 + m 4 +
+// v 4 + param 2 = 28 bytes (bf16 mode).  Each fp32 operation is rounded on its own (no FMA
+// contraction) so the result is reproducible bit for bit by a scalar CPU loop.
+#include "common.h"
+
+namespace {
+
+struct AdamScalars {
+    float b1, b2, omb1, omb2, bc1, bc2, eps, neg_lr, neg_lr_wd;
+    int use_wd;
+};
+
+#pragma clang fp contract(off)
+__device__ __forceinline__ void adam_update(float g, float &m, float &v, float &w,
+                                            const AdamScalars &s) {
+    float mm = m * s.b1;
+    mm = mm + s.omb1 * g;
+    float vv = v * s.b2;
+    vv = vv + (s.omb2 * g) * g;
+    float mh = mm / s.bc1;
+    float vh = vv / s.bc2;
+    float d = sqrtf(vh) + s.eps;
+    float ww = w + s.neg_lr * (mh / d);
+    if (s.use_wd) ww = ww + s.neg_lr_wd * ww;
+    m = mm; v = vv; w = ww;
+}
+
+template <typename V> __device__ __forceinline__ V ld_stream(const V *p) {
+    return __builtin_nontemporal_load(p);
+}
+template <typename V> __device__ __forceinline__ void st_stream(V *p, V v) {
+    __builtin_nontemporal_store(v, p);
+}
+
+// bf16 mode: a thread owns 8 consecutive elements per chunk (16 B of grad/param, 2x16 B of
+// each fp32 state); a block owns UNROLL consecutive chunks-of-256-threads so UNROLL x 7 loads
+// are in flight per thread before the first use.
+template <int UNROLL>
+__global__ __launch_bounds__(256) void adamw_bf16_kernel(uint16_t *__restrict__ param,
+                                                         const uint16_t *__restrict__ grad,
+                                                         float *__restrict__ master,
+                                                         float *__restrict__ exp_avg,
+                                                         float *__restrict__ exp_avg_sq,
+                                                         int64_t n_vec8, AdamScalars s) {
+    const int64_t base = (static_cast<int64_t>(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
+    u32x4 gq[UNROLL];
+    f32x4 m0[UNROLL], m1[UNROLL], v0[UNROLL], v1[UNROLL], w0[UNROLL], w1[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const int64_t c = base + static_cast<int64_t>(u) * 256;
+        if (c < n_vec8) {
+            gq[u] = ld_stream(reinterpret_cast<const u32x4 *>(grad) + c);
+            m0[u] = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg) + 2 * c);
+            m1[u] = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg) + 2 * c + 1);
+            v0[u] = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg_sq) + 2 * c);
+            v1[u] = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg_sq) + 2 * c + 1);
+            w0[u] = ld_stream(reinterpret_cast<const f32x4 *>(master) + 2 * c);
+            w1[u] = ld_stream(reinterpret_cast<const f32x4 *>(master) + 2 * c + 1);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const int64_t c = base + static_cast<int64_t>(u) * 256;
+        if (c < n_vec8) {
+            float g[8];
+            Elem<uint16_t>::unpack(gq[u], g);
+            float w[8];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float ma = m0[u][i], va = v0[u][i], wa = w0[u][i];
+                float mb = m1[u][i], vb = v1[u][i], wb = w1[u][i];
+                adam_update(g[i], ma, va, wa, s);
+                adam_update(g[4 + i], mb, vb, wb, s);
+                m0[u][i] = ma; v0[u][i] = va; w0[u][i] = wa;
+                m1[u][i] = mb; v1[u][i] = vb; w1[u][i] = wb;
+                w[i] = wa;
+                w[4 + i] = wb;
+            }
+            st_stream(reinterpret_cast<f32x4 *>(exp_avg) + 2 * c, m0[u]);
+            st_stream(reinterpret_cast<f32x4 *>(exp_avg) + 2 * c + 1, m1[u]);
+            st_stream(reinterpret_cast<f32x4 *>(exp_avg_sq) + 2 * c, v0[u]);
+            st_stream(reinterpret_cast<f32x4 *>(exp_avg_sq) + 2 * c + 1, v1[u]);
+            st_stream(reinterpret_cast<f32x4 *>(master) + 2 * c, w0[u]);
+            st_stream(reinterpret_cast<f32x4 *>(master) + 2 * c + 1, w1[u]);
+            st_stream(reinterpret_cast<u32x4 *>(param) + c, Elem<uint16_t>::pack(w));
+        }
+    }
+}
+
+// Elements past the last full vector of 8 (at most 7), and the whole buffer in fp32 mode's tail.
+__global__ void adamw_bf16_tail_kernel(uint16_t *param, const uint16_t *grad, float *master,
+                                       float *exp_avg, float *exp_avg_sq, int64_t start, int64_t n,
+                                       AdamScalars s) {
+    const int64_t i = start + threadIdx.x;
+    if (i < n) {
+        float m = exp_avg[i], v = exp_avg_sq[i], w = master[i];
+        adam_update(bf16_bits_to_f32(grad[i]), m, v, w, s);
+        exp_avg[i] = m; exp_avg_sq[i] = v; master[i] = w;
+        param[i] = f32_to_bf16_bits(w);
+    }
+}
+
+// fp32 mode: the parameter buffer is the master buffer (16 B read, 12 B written per element).
+template <int UNROLL>
+__global__ __launch_bounds__(256) void adamw_f32_kernel(float *__restrict__ master,
+                                                        const float *__restrict__ grad,
+                                                        float *__restrict__ exp_avg,
+                                                        float *__restrict__ exp_avg_sq,
+                                                        int64_t n_vec4, AdamScalars s) {
+    const int64_t base = (static_cast<int64_t>(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const int64_t c = base + static_cast<int64_t>(u) * 256;
+        if (c < n_vec4) {
+            f32x4 g = ld_stream(reinterpret_cast<const f32x4 *>(grad) + c);
+            f32x4 m = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg) + c);
+            f32x4 v = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg_sq) + c);
+            f32x4 w = ld_stream(reinterpret_cast<const f32x4 *>(master) + c);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float ma = m[i], va = v[i], wa = w[i];
+                adam_update(g[i], ma, va, wa, s);
+                m[i] = ma; v[i] = va; w[i] = wa;
+            }
+            st_stream(reinterpret_cast<f32x4 *>(exp_avg) + c, m);
+            st_stream(reinterpret_cast<f32x4 *>(exp_avg_sq) + c, v);
+            st_stream(reinterpret_cast<f32x4 *>(master) + c, w);
+        }
+    }
+}
+__global__ void adamw_f32_tail_kernel(float *master, const float *grad, float *exp_avg,
+                                      float *exp_avg_sq, int64_t start, int64_t n, AdamScalars s) {
+    const int64_t i = start + threadIdx.x;
+    if (i < n) {
+        float m = exp_avg[i], v = exp_avg_sq[i], w = master[i];
+        adam_update(grad[i], m, v, w, s);
+        exp_avg[i] = m; exp_avg_sq[i] = v; master[i] = w;
+    }
+}
+
+}  // namespace
+
+extern "C" int om_adamw_step(void *param, const void *grad, float *master, float *exp_avg,
+                             float *exp_avg_sq, int64_t n, double lr, double beta1, double beta2,
+                             double eps, double weight_decay, int64_t step, int param_dtype,
+                             void *stream) {
+    if (param_dtype != OM_BF16 && param_dtype != OM_F32) return OM_ERR_DTYPE;
+    if (n < 0 || step < 1) return OM_ERR_SHAPE;
+    if (n == 0) return OM_OK;
+    if (!grad || !master || !exp_avg || !exp_avg_sq) return OM_ERR_NULL;
+    if (param_dtype == OM_BF16 && !param) return OM_ERR_NULL;
+    if (!om_aligned16(grad) || !om_aligned16(master) || !om_aligned16(exp_avg) ||
+        !om_aligned16(exp_avg_sq) || (param_dtype == OM_BF16 && !om_aligned16(param)))
+        return OM_ERR_ALIGN;
+
+    // Scalars exactly as the reference forms them: Python doubles, narrowed to fp32 where they
+    // meet an fp32 tensor (optimizers.py:193-202).
+    AdamScalars s;
+    s.b1 = static_cast<float>(beta1);
+    s.b2 = static_cast<float>(beta2);
+    s.omb1 = static_cast<float>(1.0 - beta1);
+    s.omb2 = static_cast<float>(1.0 - beta2);
+    s.bc1 = static_cast<float>(1.0 - pow(beta1, static_cast<double>(step)));
+    s.bc2 = static_cast<float>(1.0 - pow(beta2, static_cast<double>(step)));
+    s.eps = static_cast<float>(eps);
+    s.neg_lr = static_cast<float>(-lr);
+    s.neg_lr_wd = static_cast<float>(-lr * weight_decay);
+    s.use_wd = weight_decay > 0.0 ? 1 : 0;
+
+    hipStream_t st = om_stream(stream);
+    constexpr int UNROLL = 2;
+    if (param_dtype == OM_BF16) {
+        const int64_t n_vec = n / 8;
+        if (n_vec > 0) {
+            const int64_t blocks = (n_vec + 256 * UNROLL - 1) / (256 * UNROLL);
+            if (blocks > 0x7fffffffLL) return OM_ERR_SHAPE;
+            adamw_bf16_kernel<UNROLL><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(
+                static_cast<uint16_t *>(param), static_cast<const uint16_t *>(grad), master, exp_avg,
+                exp_avg_sq, n_vec, s);
+        }
+        if (n_vec * 8 < n)
+            adamw_bf16_tail_kernel<<<1, 64, 0, st>>>(static_cast<uint16_t *>(param),
+                                                     static_cast<const uint16_t *>(grad), master,
+                                                     exp_avg, exp_avg_sq, n_vec * 8, n, s);
+    } else {
+        const int64_t n_vec = n / 4;
+        if (n_vec > 0) {
+            const int64_t blocks = (n_vec + 256 * UNROLL - 1) / (256 * UNROLL);
+            if (blocks > 0x7fffffffLL) return OM_ERR_SHAPE;
+            adamw_f32_kernel<UNROLL><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(
+                master, static_cast<const float *>(grad), exp_avg, exp_avg_sq, n_vec, s);
+        }
+        if (n_vec * 4 < n)
+            adamw_f32_tail_kernel<<<1, 64, 0, st>>>(master, static_cast<const float *>(grad),
+                                                    exp_avg, exp_avg_sq, n_vec * 4, n, s);
+    }
+    return om_launch_status();
+}

@@ -1,0 +1,352 @@
+// Routers: one wavefront per token.
+//  * softmax -> top-K (-> renormalise) of the OLMoE block, forward and backward;
+//  * sigmoid -> bias-corrected group-limited top-K of the DeepSeek-V3 block, forward and backward.
+// Selection order is total: (score descending, expert index ascending), so the result does not
+// depend on lane scheduling.  Scores live in registers, expert i = lane + 64*j.
+#include "common.h"
+
+namespace {
+
+#pragma clang fp contract(off)
+
+constexpr int TOKENS_PER_BLOCK = 4;
+
+template <typename T> __device__ __forceinline__ float load_logit(const T *p);
+template <> __device__ __forceinline__ float load_logit<float>(const float *p) { return *p; }
+template <> __device__ __forceinline__ float load_logit<uint16_t>(const uint16_t *p) { return bf16_bits_to_f32(*p); }
+
+// (value, index) arg-max across the wavefront; ties go to the lower index.
+__device__ __forceinline__ void wave_argmax(float &v, int &i) {
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o, 64);
+        const int oi = __shfl_xor(i, o, 64);
+        if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+    }
+}
+
+// softmax probabilities of this token's row into p[PER]; returns nothing else.
+template <int PER, typename T>
+__device__ __forceinline__ void row_softmax(const T *row, int N, int lane, float (&p)[PER]) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int i = lane + 64 * j;
+        p[j] = (i < N) ? load_logit<T>(row + i) : -INFINITY;
+        mx = fmaxf(mx, p[j]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int i = lane + 64 * j;
+        p[j] = (i < N) ? expf(p[j] - mx) : 0.0f;
+        sum += p[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < PER; j++) p[j] = p[j] / sum;
+}
+
+// K rounds of wave arg-max over s[PER] (entries with index >= N must be < every real score).
+// Lane r keeps the r-th winner in (my_v, my_i).
+template <int PER>
+__device__ __forceinline__ void select_topk(float (&s)[PER], int N, int K, int lane, float &my_v,
+                                            int &my_i) {
+    my_v = 0.0f;
+    my_i = 0;
+    for (int r = 0; r < K; r++) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const int i = lane + 64 * j;
+            if (i < N && (s[j] > bv)) { bv = s[j]; bi = i; }  // ascending i: first max wins
+        }
+        wave_argmax(bv, bi);
+        if (lane == r) { my_v = bv; my_i = bi; }
+#pragma unroll
+        for (int j = 0; j < PER; j++)
+            if (lane + 64 * j == bi) s[j] = -INFINITY;  // taken
+    }
+}
+
+template <int PER, typename T, typename TW>
+__global__ __launch_bounds__(256) void softmax_topk_kernel(const T *__restrict__ logits, int64_t Tn,
+                                                           int N, int K, int renorm,
+                                                           TW *__restrict__ weights_out,
+                                                           int64_t *__restrict__ experts_out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * TOKENS_PER_BLOCK + (threadIdx.x >> 6);
+    if (t >= Tn) return;
+    float p[PER];
+    row_softmax<PER, T>(logits + t * N, N, lane, p);
+    float w; int e;
+    select_topk<PER>(p, N, K, lane, w, e);
+    if (renorm) {
+        const float s = wave_sum(lane < K ? w : 0.0f);
+        w = w / s;
+    }
+    if (lane < K) {
+        Elem<TW>::store(weights_out + t * K + lane, w);
+        experts_out[t * K + lane] = e;
+    }
+}
+
+// dlogits_i = p_i * (dp_i - sum_j dp_j p_j), dp = scatter of dw over the selected experts, and
+// with renormalisation dw_k = (dw'_k - sum_j dw'_j w_j / S) / S, S = sum_k w_k, w_k = p[e_k].
+template <int PER, typename T, typename TW>
+__global__ __launch_bounds__(256) void softmax_topk_bwd_kernel(const T *__restrict__ logits,
+                                                               const int64_t *__restrict__ experts,
+                                                               const TW *__restrict__ dweights,
+                                                               int64_t Tn, int N, int K, int renorm,
+                                                               T *__restrict__ dlogits) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * TOKENS_PER_BLOCK + (threadIdx.x >> 6);
+    if (t >= Tn) return;
+    float p[PER];
+    row_softmax<PER, T>(logits + t * N, N, lane, p);
+    // lane k < K: its expert, the probability there and the incoming gradient
+    const int e = (lane < K) ? static_cast<int>(experts[t * K + lane]) : -1;
+    float dwk = (lane < K) ? Elem<TW>::load(dweights + t * K + lane) : 0.0f;
+    float wk = 0.0f;
+    for (int k = 0; k < K; k++) {
+        const int ek = __shfl(e, k, 64);
+        float pv = 0.0f;
+#pragma unroll
+        for (int j = 0; j < PER; j++)
+            if (lane + 64 * j == ek) pv = p[j];
+        pv = wave_sum(pv);  // exactly one lane holds it
+        if (lane == k) wk = pv;
+    }
+    if (renorm) {
+        const float S = wave_sum(wk);
+        const float dot = wave_sum(dwk * wk);
+        dwk = (dwk - dot / S) / S;
+    }
+    const float inner = wave_sum(dwk * wk);  // sum_j dp_j p_j
+    float dp[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) dp[j] = 0.0f;
+    for (int k = 0; k < K; k++) {
+        const int ek = __shfl(e, k, 64);
+        const float dk = __shfl(dwk, k, 64);
+#pragma unroll
+        for (int j = 0; j < PER; j++)
+            if (lane + 64 * j == ek) dp[j] = dk;
+    }
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int i = lane + 64 * j;
+        if (i < N) Elem<T>::store(dlogits + t * N + i, p[j] * (dp[j] - inner));
+    }
+}
+
+// DeepSeek-V3 group-limited routing.  LDS holds the choice scores of the 4 tokens of the block
+// so a lane can scan "its" group; everything else stays in registers.
+template <int PER>
+__global__ __launch_bounds__(256) void sigmoid_group_topk_kernel(
+    const float *__restrict__ logits, const float *__restrict__ bias, int64_t Tn, int N, int n_group,
+    int topk_group, int K, int renorm, float scale, int64_t *__restrict__ experts_out,
+    float *__restrict__ weights_out) {
+    __shared__ float choice_lds[TOKENS_PER_BLOCK][PER * 64];
+    const int lane = threadIdx.x & 63;
+    const int wv = threadIdx.x >> 6;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * TOKENS_PER_BLOCK + wv;
+    if (t >= Tn) return;  // whole wavefront leaves together; no block-wide barrier below
+    float score[PER], choice[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int i = lane + 64 * j;
+        if (i < N) {
+            const float x = logits[t * N + i];
+            score[j] = 1.0f / (1.0f + expf(-x));
+            choice[j] = score[j] + bias[i];
+            choice_lds[wv][i] = choice[j];
+        } else {
+            score[j] = 0.0f;
+            choice[j] = -INFINITY;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // lane g < n_group: sum of the two largest choice values of group g
+    const int gs = N / n_group;
+    float gscore = -INFINITY;
+    if (lane < n_group) {
+        float a = -INFINITY, b = -INFINITY;
+        for (int i = 0; i < gs; i++) {
+            const float v = choice_lds[wv][lane * gs + i];
+            if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+        }
+        gscore = (gs >= 2) ? (a + b) : a;
+    }
+    // keep the topk_group best groups (score desc, group index asc)
+    unsigned long long keep = 0ull;
+    for (int r = 0; r < topk_group; r++) {
+        float bv = gscore; int bi = (lane < n_group) ? lane : 0x7fffffff;
+        wave_argmax(bv, bi);
+        keep |= (1ull << bi);
+        if (lane == bi) gscore = -INFINITY;
+    }
+    // masked_fill(~mask, 0.0): dropped groups compete with the value 0.0
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int i = lane + 64 * j;
+        if (i < N && !((keep >> (i / gs)) & 1ull)) choice[j] = 0.0f;
+    }
+    float cv; int e;
+    select_topk<PER>(choice, N, K, lane, cv, e);
+    // weight = sigmoid score (no bias) at the selected expert
+    float w = 0.0f;
+    for (int k = 0; k < K; k++) {
+        const int ek = __shfl(e, k, 64);
+        float sv = 0.0f;
+#pragma unroll
+        for (int j = 0; j < PER; j++)
+            if (lane + 64 * j == ek) sv = score[j];
+        sv = wave_sum(sv);
+        if (lane == k) w = sv;
+    }
+    if (renorm) {
+        const float S = wave_sum(lane < K ? w : 0.0f) + 1e-20f;
+        w = w / S;
+    }
+    w = w * scale;
+    if (lane < K) {
+        experts_out[t * K + lane] = e;
+        weights_out[t * K + lane] = w;
+    }
+}
+
+// w'_k = scale * s_k / (S + 1e-20) (or scale * s_k); ds_k -> dlogit = ds * s * (1 - s).
+template <int PER>
+__global__ __launch_bounds__(256) void sigmoid_topk_bwd_kernel(const float *__restrict__ logits,
+                                                               const int64_t *__restrict__ experts,
+                                                               const float *__restrict__ dweights,
+                                                               int64_t Tn, int N, int K, int renorm,
+                                                               float scale, float *__restrict__ dlogits) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * TOKENS_PER_BLOCK + (threadIdx.x >> 6);
+    if (t >= Tn) return;
+    const int e = (lane < K) ? static_cast<int>(experts[t * K + lane]) : -1;
+    float sk = 0.0f;
+    if (lane < K) sk = 1.0f / (1.0f + expf(-logits[t * N + e]));
+    float d = (lane < K) ? dweights[t * K + lane] * scale : 0.0f;  // through "* scale"
+    if (renorm) {
+        const float S = wave_sum(sk) + 1e-20f;
+        const float dot = wave_sum(d * sk);
+        d = (d - dot / S) / S;
+    }
+    const float dl = d * (sk * (1.0f - sk));
+    float out[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) out[j] = 0.0f;
+    for (int k = 0; k < K; k++) {
+        const int ek = __shfl(e, k, 64);
+        const float dk = __shfl(dl, k, 64);
+#pragma unroll
+        for (int j = 0; j < PER; j++)
+            if (lane + 64 * j == ek) out[j] += dk;
+    }
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int i = lane + 64 * j;
+        if (i < N) dlogits[t * N + i] = out[j];
+    }
+}
+
+inline unsigned token_blocks(int64_t T) {
+    return static_cast<unsigned>((T + TOKENS_PER_BLOCK - 1) / TOKENS_PER_BLOCK);
+}
+inline int per_lane(int N) { return N <= 64 ? 1 : N <= 128 ? 2 : N <= 256 ? 4 : 8; }
+
+}  // namespace
+
+#define OM_DISPATCH_PER(N, CALL)              \
+    switch (per_lane(N)) {                    \
+        case 1: { constexpr int PER = 1; CALL; } break; \
+        case 2: { constexpr int PER = 2; CALL; } break; \
+        case 4: { constexpr int PER = 4; CALL; } break; \
+        default: { constexpr int PER = 8; CALL; } break; \
+    }
+
+extern "C" int om_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int N, int K,
+                                     int norm_topk_prob, void *weights_out, int weights_dtype,
+                                     int64_t *experts_out, void *stream) {
+    if ((logits_dtype != OM_F32 && logits_dtype != OM_BF16) ||
+        (weights_dtype != OM_F32 && weights_dtype != OM_BF16))
+        return OM_ERR_DTYPE;
+    if (T < 0 || N < 1 || N > 512 || K < 1 || K > N || K > 64 || T > 0x7fffffffLL) return OM_ERR_SHAPE;
+    if (T == 0) return OM_OK;
+    if (!logits || !weights_out || !experts_out) return OM_ERR_NULL;
+    hipStream_t st = om_stream(stream);
+    const unsigned nb = token_blocks(T);
+#define OM_RT(TL, TW)                                                                          \
+    OM_DISPATCH_PER(N, (softmax_topk_kernel<PER, TL, TW><<<nb, 256, 0, st>>>(                  \
+                           static_cast<const TL *>(logits), T, N, K, norm_topk_prob,           \
+                           static_cast<TW *>(weights_out), experts_out)))
+    if (logits_dtype == OM_F32 && weights_dtype == OM_F32) { OM_RT(float, float); }
+    else if (logits_dtype == OM_F32) { OM_RT(float, uint16_t); }
+    else if (weights_dtype == OM_F32) { OM_RT(uint16_t, float); }
+    else { OM_RT(uint16_t, uint16_t); }
+#undef OM_RT
+    return om_launch_status();
+}
+
+extern "C" int om_route_softmax_topk_bwd(const void *logits, int logits_dtype, const int64_t *experts,
+                                         const void *dweights, int weights_dtype, int64_t T, int N,
+                                         int K, int norm_topk_prob, void *dlogits, void *stream) {
+    if ((logits_dtype != OM_F32 && logits_dtype != OM_BF16) ||
+        (weights_dtype != OM_F32 && weights_dtype != OM_BF16))
+        return OM_ERR_DTYPE;
+    if (T < 0 || N < 1 || N > 512 || K < 1 || K > N || K > 64 || T > 0x7fffffffLL) return OM_ERR_SHAPE;
+    if (T == 0) return OM_OK;
+    if (!logits || !experts || !dweights || !dlogits) return OM_ERR_NULL;
+    hipStream_t st = om_stream(stream);
+    const unsigned nb = token_blocks(T);
+#define OM_RB(TL, TW)                                                                          \
+    OM_DISPATCH_PER(N, (softmax_topk_bwd_kernel<PER, TL, TW><<<nb, 256, 0, st>>>(              \
+                           static_cast<const TL *>(logits), experts,                           \
+                           static_cast<const TW *>(dweights), T, N, K, norm_topk_prob,         \
+                           static_cast<TL *>(dlogits))))
+    if (logits_dtype == OM_F32 && weights_dtype == OM_F32) { OM_RB(float, float); }
+    else if (logits_dtype == OM_F32) { OM_RB(float, uint16_t); }
+    else if (weights_dtype == OM_F32) { OM_RB(uint16_t, float); }
+    else { OM_RB(uint16_t, uint16_t); }
+#undef OM_RB
+    return om_launch_status();
+}
+
+extern "C" int om_route_sigmoid_group_topk(const float *logits, const float *bias, int64_t T, int N,
+                                           int n_group, int topk_group, int K, int norm_topk_prob,
+                                           double routed_scaling_factor, int64_t *experts_out,
+                                           float *weights_out, void *stream) {
+    if (T < 0 || N < 1 || N > 512 || K < 1 || K > N || K > 64 || n_group < 1 || n_group > 64 ||
+        N % n_group != 0 || topk_group < 1 || topk_group > n_group || T > 0x7fffffffLL)
+        return OM_ERR_SHAPE;
+    if (T == 0) return OM_OK;
+    if (!logits || !bias || !experts_out || !weights_out) return OM_ERR_NULL;
+    hipStream_t st = om_stream(stream);
+    const unsigned nb = token_blocks(T);
+    const float scale = static_cast<float>(routed_scaling_factor);
+    OM_DISPATCH_PER(N, (sigmoid_group_topk_kernel<PER><<<nb, 256, 0, st>>>(
+                           logits, bias, T, N, n_group, topk_group, K, norm_topk_prob, scale,
+                           experts_out, weights_out)));
+    return om_launch_status();
+}
+
+extern "C" int om_route_sigmoid_topk_bwd(const float *logits, const int64_t *experts,
+                                         const float *dweights, int64_t T, int N, int K,
+                                         int norm_topk_prob, double routed_scaling_factor,
+                                         float *dlogits, void *stream) {
+    if (T < 0 || N < 1 || N > 512 || K < 1 || K > N || K > 64 || T > 0x7fffffffLL) return OM_ERR_SHAPE;
+    if (T == 0) return OM_OK;
+    if (!logits || !experts || !dweights || !dlogits) return OM_ERR_NULL;
+    hipStream_t st = om_stream(stream);
+    const unsigned nb = token_blocks(T);
+    const float scale = static_cast<float>(routed_scaling_factor);
+    OM_DISPATCH_PER(N, (sigmoid_topk_bwd_kernel<PER><<<nb, 256, 0, st>>>(
+                           logits, experts, dweights, T, N, K, norm_topk_prob, scale, dlogits)));
+    return om_launch_status();
+}

@@ -1,0 +1,338 @@
+// Token permutation for the fast MoE block: a stable counting sort of the (token, k) pairs by
+// local expert, producing exactly the arrays the reference builds with its two index kernels and
+// two cumsums.  Three small launches:
+//   count   — every block histograms its chunk of pairs per expert (wave ballots -> LDS);
+//   scan    — one block turns the [block][expert] table into exclusive offsets in
+//             (expert-major, block-minor) order = the stable order, and writes cum_token_counts;
+//   scatter — every block re-reads its chunk and places each pair at offset + stable rank.
+// Ranks come from wavefront ballots (lanes holding the same expert form a mask; rank = popcount of
+// the mask below the lane), per-wave running offsets live in LDS: no atomics, so the result is
+// deterministic.
+// Also: the reference's two index kernels with their own [expert][column] table layout.
+#include "common.h"
+
+namespace {
+
+constexpr int SORT_THREADS = 256;
+constexpr int SORT_WAVES = SORT_THREADS / 64;
+constexpr int SORT_ITERS = 8;                                    // 64-pair steps per wavefront
+constexpr int SORT_CHUNK = SORT_THREADS * SORT_ITERS;            // pairs per block
+constexpr int SORT_MAX_NR = 1024;                                // local experts supported
+
+template <typename TI>
+__device__ __forceinline__ int local_key(const TI *selected_experts, int64_t j, int64_t n_pairs,
+                                         int start, int end, int NR) {
+    if (j >= n_pairs) return NR;
+    const long long e = static_cast<long long>(selected_experts[j]);
+    return (e >= start && e < end) ? static_cast<int>(e - start) : NR;
+}
+
+// Mask of the lanes of this wavefront that hold the same key (keys < 2^nbits).
+__device__ __forceinline__ unsigned long long match_key(int key, int nbits) {
+    unsigned long long m = ~0ull;
+    for (int b = 0; b < nbits; b++) {
+        const unsigned long long vote = __ballot((key >> b) & 1);
+        m &= ((key >> b) & 1) ? vote : ~vote;
+    }
+    return m;
+}
+
+__device__ __forceinline__ unsigned long long lanemask_lt(int lane) { return (1ull << lane) - 1ull; }
+
+// Per-wave histogram of the wave's SORT_ITERS*64 pairs into wave_hist[wave][0..NR).
+template <typename TI>
+__device__ __forceinline__ int wave_histogram(const TI *selected_experts, int64_t wave_base,
+                                              int64_t n_pairs, int start, int end, int NR, int nbits,
+                                              int lane, volatile int *hist) {
+    int hits = 0;
+    for (int it = 0; it < SORT_ITERS; it++) {
+        const int64_t j = wave_base + it * 64 + lane;
+        const int key = local_key(selected_experts, j, n_pairs, start, end, NR);
+        const unsigned long long m = match_key(key, nbits);
+        const bool leader = (__ffsll(static_cast<long long>(m)) - 1) == lane;
+        if (leader && key < NR) hist[key] += __popcll(m);
+        hits += __popcll(__ballot(key < NR));
+        __builtin_amdgcn_wave_barrier();
+    }
+    return hits;
+}
+
+template <typename TI>
+__global__ __launch_bounds__(SORT_THREADS) void sort_count_kernel(const TI *__restrict__ selected_experts,
+                                                                  int64_t n_pairs, int start, int end,
+                                                                  int NR, int nbits,
+                                                                  int32_t *__restrict__ block_hist) {
+    extern __shared__ int lds[];  // [SORT_WAVES][NR]
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < SORT_WAVES * NR; i += SORT_THREADS) lds[i] = 0;
+    __syncthreads();
+    const int64_t wave_base = static_cast<int64_t>(blockIdx.x) * SORT_CHUNK + wv * (SORT_ITERS * 64);
+    wave_histogram(selected_experts, wave_base, n_pairs, start, end, NR, nbits, lane, lds + wv * NR);
+    __syncthreads();
+    for (int e = threadIdx.x; e < NR; e += SORT_THREADS) {
+        int s = 0;
+        for (int w = 0; w < SORT_WAVES; w++) s += lds[w * NR + e];
+        block_hist[static_cast<int64_t>(blockIdx.x) * NR + e] = s;
+    }
+}
+
+// One block.  block_hist [NB][NR] -> in place: exclusive offset of (expert e, block b) in the
+// stable order; hits_base [NB] = pairs kept by blocks before b; cum_token_counts [NR+1].
+__global__ __launch_bounds__(1024) void sort_scan_kernel(int32_t *__restrict__ block_hist,
+                                                          int32_t *__restrict__ hits_base, int NB,
+                                                          int NR, int32_t *__restrict__ cum_token_counts,
+                                                          int32_t *__restrict__ cum_expert_counts_ep,
+                                                          int64_t T) {
+    __shared__ int totals[SORT_MAX_NR + 1];
+    // per-expert exclusive scan over blocks
+    for (int e = threadIdx.x; e < NR; e += blockDim.x) {
+        int run = 0;
+        for (int b = 0; b < NB; b++) {
+            const int c = block_hist[static_cast<int64_t>(b) * NR + e];
+            block_hist[static_cast<int64_t>(b) * NR + e] = run;
+            run += c;
+        }
+        totals[e] = run;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {  // NR <= 1024: a serial scan is a microsecond
+        int run = 0;
+        for (int e = 0; e < NR; e++) {
+            const int c = totals[e];
+            totals[e] = run;
+            cum_token_counts[e] = run;
+            run += c;
+        }
+        totals[NR] = run;
+        cum_token_counts[NR] = run;
+        cum_expert_counts_ep[T] = run;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < NR; e += blockDim.x) {
+        const int base = totals[e];
+        for (int b = 0; b < NB; b++) block_hist[static_cast<int64_t>(b) * NR + e] += base;
+    }
+    // pairs kept per block = offset(e, b+1) - offset(e, b) summed over e; recompute from the
+    // offsets just written: kept(b) = sum_e (off[b+1][e] - off[b][e]) with off[NB][e] = totals[e+1].
+    __syncthreads();
+    for (int b = threadIdx.x; b < NB; b += blockDim.x) {
+        int kept_before = 0;  // pairs of blocks < b = sum_e (off[b][e] - totals[e])
+        for (int e = 0; e < NR; e++) kept_before += block_hist[static_cast<int64_t>(b) * NR + e] - totals[e];
+        hits_base[b] = kept_before;
+    }
+}
+
+template <typename TI>
+__global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(
+    const TI *__restrict__ selected_experts, int64_t n_pairs, int K, int start, int end, int NR,
+    int nbits, const int32_t *__restrict__ block_offsets, const int32_t *__restrict__ hits_base,
+    int32_t *__restrict__ cum_expert_counts_ep, int32_t *__restrict__ input_indices,
+    int32_t *__restrict__ output_indices, int32_t *__restrict__ selected_experts_indices) {
+    extern __shared__ int lds[];  // [SORT_WAVES][NR] then [SORT_WAVES] wave hit counts
+    int *wave_hits = lds + SORT_WAVES * NR;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < SORT_WAVES * NR; i += SORT_THREADS) lds[i] = 0;
+    __syncthreads();
+    const int64_t wave_base = static_cast<int64_t>(blockIdx.x) * SORT_CHUNK + wv * (SORT_ITERS * 64);
+    const int hits = wave_histogram(selected_experts, wave_base, n_pairs, start, end, NR, nbits, lane,
+                                    lds + wv * NR);
+    if (lane == 0) wave_hits[wv] = hits;
+    __syncthreads();
+    // counts -> running offsets: off[w][e] = block offset + counts of the waves before w
+    for (int e = threadIdx.x; e < NR; e += SORT_THREADS) {
+        int run = block_offsets[static_cast<int64_t>(blockIdx.x) * NR + e];
+        for (int w = 0; w < SORT_WAVES; w++) {
+            const int c = lds[w * NR + e];
+            lds[w * NR + e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    int oi_base = hits_base[blockIdx.x];
+    for (int w = 0; w < wv; w++) oi_base += wave_hits[w];
+    volatile int *off = lds + wv * NR;
+    for (int it = 0; it < SORT_ITERS; it++) {
+        const int64_t j = wave_base + it * 64 + lane;
+        const int key = local_key(selected_experts, j, n_pairs, start, end, NR);
+        const unsigned long long m = match_key(key, nbits);
+        const unsigned long long kept = __ballot(key < NR);
+        const int oi = oi_base + __popcll(kept & lanemask_lt(lane));
+        const bool valid = j < n_pairs;
+        const int64_t t = valid ? j / K : 0;
+        const int k = valid ? static_cast<int>(j - t * K) : 0;
+        if (valid && k == 0) cum_expert_counts_ep[t] = oi;
+        if (key < NR) {
+            const int pos = off[key] + __popcll(m & lanemask_lt(lane));
+            __builtin_amdgcn_wave_barrier();
+            const bool leader = (__ffsll(static_cast<long long>(m)) - 1) == lane;
+            if (leader) off[key] += __popcll(m);
+            input_indices[pos] = static_cast<int32_t>(t);
+            output_indices[oi] = pos;
+            selected_experts_indices[oi] = k;
+        } else {
+            __builtin_amdgcn_wave_barrier();
+        }
+        oi_base += __popcll(kept);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+inline int key_bits(int NR) {  // keys 0..NR (NR = "not local")
+    int b = 1;
+    while ((1 << b) <= NR) b++;
+    return b;
+}
+
+// ---- the reference's own index kernels (table layout [expert][column]) -----------------------
+template <typename TI>
+__global__ void partial_token_counts_kernel(const TI *__restrict__ selected_experts,
+                                            int32_t *__restrict__ partial_token_counts,
+                                            int32_t *__restrict__ expert_counts_ep, int start, int end,
+                                            int K, int64_t TB, int64_t TH) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (tid >= TH) return;
+    for (int64_t lt = 0; lt < TB; lt++) {
+        int expert_count = 0;
+        const int64_t t = tid * TB + lt;
+        for (int k = 0; k < K; k++) {
+            const long long n = static_cast<long long>(selected_experts[t * K + k]);
+            if (n >= start && n < end) {
+                partial_token_counts[(n - start) * TH + tid] += 1;
+                expert_count += 1;
+            }
+        }
+        expert_counts_ep[t] = expert_count;
+    }
+}
+
+template <typename TI>
+__global__ void input_and_output_indices_kernel(
+    const TI *__restrict__ selected_experts, const int32_t *__restrict__ partial_cum_token_counts,
+    int32_t *__restrict__ input_increment_buffer, const int32_t *__restrict__ cum_expert_counts_ep,
+    int32_t *__restrict__ selected_experts_indices, int32_t *__restrict__ input_indices,
+    int32_t *__restrict__ output_indices, int start, int end, int K, int64_t TB, int64_t TH) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (tid >= TH) return;
+    for (int64_t t = tid * TB; t < (tid + 1) * TB; t++) {
+        int output_index = cum_expert_counts_ep[t];
+        for (int k = 0; k < K; k++) {
+            const long long n = static_cast<long long>(selected_experts[t * K + k]);
+            if (n >= start && n < end) {
+                const int64_t cell = (n - start) * TH + tid;
+                const int offset = input_increment_buffer[cell];
+                const int input_index = partial_cum_token_counts[cell] + offset;
+                input_indices[input_index] = static_cast<int32_t>(t);
+                input_increment_buffer[cell] = offset + 1;
+                output_indices[output_index] = input_index;
+                selected_experts_indices[output_index] = k;
+                output_index += 1;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int64_t om_moe_sort_workspace_bytes(int64_t T, int K, int NR) {
+    if (T < 0 || K < 1 || NR < 1) return 0;
+    const int64_t n_pairs = T * K;
+    const int64_t NB = (n_pairs + SORT_CHUNK - 1) / SORT_CHUNK;
+    return (NB * NR + NB + 1) * static_cast<int64_t>(sizeof(int32_t));
+}
+
+extern "C" int om_moe_sort(const void *selected_experts, int index_dtype, int64_t T, int K,
+                           int expert_start_idx, int expert_end_idx, int32_t *cum_token_counts,
+                           int32_t *cum_expert_counts_ep, int32_t *input_indices,
+                           int32_t *output_indices, int32_t *selected_experts_indices,
+                           void *workspace, int64_t workspace_bytes, void *stream) {
+    if (index_dtype != OM_I32 && index_dtype != OM_I64) return OM_ERR_DTYPE;
+    const int NR = expert_end_idx - expert_start_idx;
+    if (T < 0 || K < 1 || NR < 1 || NR > SORT_MAX_NR || expert_start_idx < 0) return OM_ERR_SHAPE;
+    const int64_t n_pairs = T * K;
+    if (n_pairs > 0x7fffffffLL) return OM_ERR_SHAPE;
+    if (!cum_token_counts || !cum_expert_counts_ep) return OM_ERR_NULL;
+    if (T > 0 && (!selected_experts || !input_indices || !output_indices || !selected_experts_indices))
+        return OM_ERR_NULL;
+    const int64_t NB = (n_pairs + SORT_CHUNK - 1) / SORT_CHUNK;
+    if (workspace_bytes < om_moe_sort_workspace_bytes(T, K, NR)) return OM_ERR_WORKSPACE;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 3u)) return OM_ERR_ALIGN;
+    int32_t *block_hist = static_cast<int32_t *>(workspace);
+    int32_t *hits_base = block_hist + NB * NR;
+    hipStream_t st = om_stream(stream);
+    const int nbits = key_bits(NR);
+    const size_t lds_count = static_cast<size_t>(SORT_WAVES) * NR * sizeof(int);
+    const size_t lds_scatter = lds_count + SORT_WAVES * sizeof(int);
+    if (NB > 0) {
+        if (index_dtype == OM_I64)
+            sort_count_kernel<int64_t><<<static_cast<unsigned>(NB), SORT_THREADS, lds_count, st>>>(
+                static_cast<const int64_t *>(selected_experts), n_pairs, expert_start_idx,
+                expert_end_idx, NR, nbits, block_hist);
+        else
+            sort_count_kernel<int32_t><<<static_cast<unsigned>(NB), SORT_THREADS, lds_count, st>>>(
+                static_cast<const int32_t *>(selected_experts), n_pairs, expert_start_idx,
+                expert_end_idx, NR, nbits, block_hist);
+    }
+    sort_scan_kernel<<<1, 1024, 0, st>>>(block_hist, hits_base, static_cast<int>(NB), NR,
+                                         cum_token_counts, cum_expert_counts_ep, T);
+    if (NB > 0) {
+        if (index_dtype == OM_I64)
+            sort_scatter_kernel<int64_t><<<static_cast<unsigned>(NB), SORT_THREADS, lds_scatter, st>>>(
+                static_cast<const int64_t *>(selected_experts), n_pairs, K, expert_start_idx,
+                expert_end_idx, NR, nbits, block_hist, hits_base, cum_expert_counts_ep, input_indices,
+                output_indices, selected_experts_indices);
+        else
+            sort_scatter_kernel<int32_t><<<static_cast<unsigned>(NB), SORT_THREADS, lds_scatter, st>>>(
+                static_cast<const int32_t *>(selected_experts), n_pairs, K, expert_start_idx,
+                expert_end_idx, NR, nbits, block_hist, hits_base, cum_expert_counts_ep, input_indices,
+                output_indices, selected_experts_indices);
+    }
+    return om_launch_status();
+}
+
+extern "C" int om_compute_partial_token_counts(const void *selected_experts, int index_dtype,
+                                               int32_t *partial_token_counts,
+                                               int32_t *expert_counts_ep, int expert_start_idx,
+                                               int expert_end_idx, int64_t T, int K, int64_t TH,
+                                               void *stream) {
+    if (index_dtype != OM_I32 && index_dtype != OM_I64) return OM_ERR_DTYPE;
+    if (T < 0 || K < 1 || TH < 1 || T % TH != 0) return OM_ERR_SHAPE;
+    if (T == 0) return OM_OK;
+    if (!selected_experts || !partial_token_counts || !expert_counts_ep) return OM_ERR_NULL;
+    hipStream_t st = om_stream(stream);
+    const unsigned nb = static_cast<unsigned>((TH + 63) / 64);
+    if (index_dtype == OM_I64)
+        partial_token_counts_kernel<int64_t><<<nb, 64, 0, st>>>(
+            static_cast<const int64_t *>(selected_experts), partial_token_counts, expert_counts_ep,
+            expert_start_idx, expert_end_idx, K, T / TH, TH);
+    else
+        partial_token_counts_kernel<int32_t><<<nb, 64, 0, st>>>(
+            static_cast<const int32_t *>(selected_experts), partial_token_counts, expert_counts_ep,
+            expert_start_idx, expert_end_idx, K, T / TH, TH);
+    return om_launch_status();
+}
+
+extern "C" int om_compute_input_and_output_indices(
+    const void *selected_experts, int index_dtype, const int32_t *partial_cum_token_counts,
+    int32_t *input_increment_buffer, const int32_t *cum_expert_counts_ep,
+    int32_t *selected_experts_indices, int32_t *input_indices, int32_t *output_indices,
+    int expert_start_idx, int expert_end_idx, int64_t T, int K, int64_t TH, void *stream) {
+    if (index_dtype != OM_I32 && index_dtype != OM_I64) return OM_ERR_DTYPE;
+    if (T < 0 || K < 1 || TH < 1 || T % TH != 0) return OM_ERR_SHAPE;
+    if (T == 0) return OM_OK;
+    if (!selected_experts || !partial_cum_token_counts || !input_increment_buffer ||
+        !cum_expert_counts_ep || !selected_experts_indices || !input_indices || !output_indices)
+        return OM_ERR_NULL;
+    hipStream_t st = om_stream(stream);
+    const unsigned nb = static_cast<unsigned>((TH + 63) / 64);
+    if (index_dtype == OM_I64)
+        input_and_output_indices_kernel<int64_t><<<nb, 64, 0, st>>>(
+            static_cast<const int64_t *>(selected_experts), partial_cum_token_counts,
+            input_increment_buffer, cum_expert_counts_ep, selected_experts_indices, input_indices,
+            output_indices, expert_start_idx, expert_end_idx, K, T / TH, TH);
+    else
+        input_and_output_indices_kernel<int32_t><<<nb, 64, 0, st>>>(
+            static_cast<const int32_t *>(selected_experts), partial_cum_token_counts,
+            input_increment_buffer, cum_expert_counts_ep, selected_experts_indices, input_indices,
+            output_indices, expert_start_idx, expert_end_idx, K, T / TH, TH);
+    return om_launch_status();
+}

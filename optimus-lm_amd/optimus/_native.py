@@ -1,0 +1,134 @@
+"""ctypes binding of liboptimus_mi355x.so, the C-ABI library of HIP kernels.
+
+This is the only place that touches the library.  Tensors are passed as raw device pointers
+(`tensor.data_ptr()`), the stream is PyTorch's current HIP stream.  There is no fallback: if
+the library is missing or a call returns an error code, an exception is raised.
+"""
+import ctypes
+import os
+
+import torch
+
+_PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG_ROOT, "lib", "liboptimus_mi355x.so")
+
+OM_F32, OM_BF16 = 0, 1
+OM_I32, OM_I64 = 0, 1
+
+c_void_p = ctypes.c_void_p
+c_int = ctypes.c_int
+c_i64 = ctypes.c_int64
+c_double = ctypes.c_double
+
+# name -> (restype, argtypes); mirrors include/optimus_mi355x.h one to one
+SIGNATURES = {
+    "om_version": (c_int, []),
+    "om_arch": (ctypes.c_char_p, []),
+    "om_strerror": (ctypes.c_char_p, [c_int]),
+    "om_adamw_step": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_double,
+                              c_double, c_double, c_double, c_double, c_i64, c_int, c_void_p]),
+    "om_route_softmax_topk": (c_int, [c_void_p, c_int, c_i64, c_int, c_int, c_int, c_void_p, c_int,
+                                      c_void_p, c_void_p]),
+    "om_route_softmax_topk_bwd": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_i64, c_int,
+                                          c_int, c_int, c_void_p, c_void_p]),
+    "om_route_sigmoid_group_topk": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_int, c_int,
+                                            c_int, c_double, c_void_p, c_void_p, c_void_p]),
+    "om_route_sigmoid_topk_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int, c_int,
+                                          c_double, c_void_p, c_void_p]),
+    "om_moe_sort_workspace_bytes": (c_i64, [c_i64, c_int, c_int]),
+    "om_moe_sort": (c_int, [c_void_p, c_int, c_i64, c_int, c_int, c_int, c_void_p, c_void_p,
+                            c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_void_p]),
+    "om_compute_partial_token_counts": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
+                                                c_i64, c_int, c_i64, c_void_p]),
+    "om_compute_input_and_output_indices": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                                    c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                                    c_i64, c_int, c_i64, c_void_p]),
+    "om_index_add": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int, c_void_p]),
+    "om_index_gather": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int, c_void_p]),
+    "om_shuffle_sub_matrix_reduce": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64,
+                                             c_int, c_void_p]),
+    "om_reduce_ggemm_output": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       c_i64, c_int, c_i64, c_int, c_int, c_int, c_void_p]),
+    "om_reduce_ggemm_output_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                c_void_p, c_void_p, c_void_p, c_i64, c_int, c_i64,
+                                                c_int, c_int, c_void_p]),
+    "om_grouped_gemm_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
+                                    c_int, c_i64, c_void_p]),
+    "om_grouped_gemm_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
+                                      c_int, c_i64, c_void_p]),
+    "om_grouped_gemm_wgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
+                                      c_int, c_i64, c_void_p]),
+    "om_merged_mlp_gate_up_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_void_p, c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
+    "om_merged_mlp_down_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
+    "om_merged_mlp_gate_up_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
+    "om_swiglu_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_int, c_void_p]),
+    "om_swiglu_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int,
+                              c_void_p]),
+}
+
+_lib = None
+
+
+class NativeLibraryError(RuntimeError):
+    pass
+
+
+def lib():
+    """Load the library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise NativeLibraryError(
+                f"{LIB_PATH} not found: build it with `python optimus-lm_amd/build.py` "
+                "(there is no non-HIP fallback)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(code, what):
+    if code != 0:
+        msg = lib().om_strerror(code).decode()
+        raise NativeLibraryError(f"{what} failed with code {code}: {msg}")
+
+
+def dtype_code(t):
+    if t.dtype == torch.float32:
+        return OM_F32
+    if t.dtype == torch.bfloat16:
+        return OM_BF16
+    raise TypeError(f"unsupported dtype {t.dtype}: the HIP kernels take float32 or bfloat16")
+
+
+def index_code(t):
+    if t.dtype == torch.int64:
+        return OM_I64
+    if t.dtype == torch.int32:
+        return OM_I32
+    raise TypeError(f"expert indices must be int64 or int32, got {t.dtype}")
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def require_cuda_contiguous(*tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise NativeLibraryError("the HIP kernels need device tensors (got a CPU tensor); "
+                                     "there is no CPU fallback")
+        if not t.is_contiguous():
+            raise NativeLibraryError("the HIP kernels need contiguous row-major tensors")

@@ -1,0 +1,509 @@
+"""optimus.models.common.moe — the fast MoE block, same interface as the reference
+(optimus/models/common/moe.py:43-632), computed by the HIP kernels of liboptimus_mi355x.so.
+
+Pipeline of FastOlmoeParallelSparseMoeBlock.forward (reference moe.py:454-621):
+  router (softmax -> top-K -> optional renorm)     one wavefront per token          [route.hip]
+  K1+K2+K3 index construction                      stable counting sort on device   [sort.hip]
+  K4 gather rows into expert order                                                   [rows.hip]
+  K5 merged-MLP grouped SwiGLU GEMMs               bf16 MFMA, variable rows/expert  [ggemm.hip]
+  K6 weighted combine back to token order                                            [rows.hip]
+and the mirrored backward.  There is one code path: the reference's `use_triton_path_*` and
+`use_ref_path_*` switches are accepted where its signatures have them and ignored.
+"""
+import torch
+import torch.nn as nn
+from torch.utils.checkpoint import checkpoint as torch_activation_checkpoint
+
+import pcl_xpu_customops
+from optimus import _native as _n
+from optimus.profilers import record_pcl_function
+
+
+def get_tensor_list(tensor, cum_token_counts):
+    """Per-expert row slices (reference moe.py:28-35); host-side helper, needs CPU-readable counts."""
+    N = len(cum_token_counts) - 1
+    return [tensor[cum_token_counts[n]:cum_token_counts[n + 1]] for n in range(N)]
+
+
+def _device_counts(cum_token_counts, device):
+    """The reference hands MergedMLP a CPU int32 tensor (moe.py:494); the kernels read the counts
+    from device memory, so accept either and never read them back."""
+    if cum_token_counts.device != device:
+        cum_token_counts = cum_token_counts.to(device, non_blocking=True)
+    if cum_token_counts.dtype != torch.int32:
+        cum_token_counts = cum_token_counts.to(torch.int32)
+    return cum_token_counts.contiguous()
+
+
+def _expert_stride(weight):
+    """Elements between consecutive experts of a [G, out, in] weight whose inner two dims are
+    dense; 0 for the packed layout."""
+    G, o, i = weight.shape
+    if weight.stride(2) != 1 or weight.stride(1) != i:
+        raise _n.NativeLibraryError("expert weights must be dense [out, in] matrices")
+    s = weight.stride(0) if G > 1 else o * i
+    return 0 if s == o * i else s
+
+
+def _require_bf16(*tensors):
+    for t in tensors:
+        if t.dtype != torch.bfloat16:
+            raise TypeError(f"the grouped expert GEMMs run in bfloat16 (got {t.dtype}); cast the "
+                            "module with .to(torch.bfloat16)")
+
+
+# ----------------------------------------------------------------------------------------------
+# Router
+# ----------------------------------------------------------------------------------------------
+class SoftmaxTopkRouterFunction(torch.autograd.Function):
+    """routing_weights, selected_experts = topk(softmax_fp32(logits), K) [/ sum] -> out dtype.
+
+    Reference moe.py:467-471.  Selection order is (probability desc, expert index asc)."""
+
+    @staticmethod
+    def forward(ctx, router_logits, top_k, norm_topk_prob, out_dtype):
+        _n.require_cuda_contiguous(router_logits)
+        T, N = router_logits.shape
+        weights = torch.empty((T, top_k), dtype=out_dtype, device=router_logits.device)
+        experts = torch.empty((T, top_k), dtype=torch.int64, device=router_logits.device)
+        _n.check(_n.lib().om_route_softmax_topk(
+            _n.ptr(router_logits), _n.dtype_code(router_logits), T, N, top_k, int(bool(norm_topk_prob)),
+            _n.ptr(weights), _n.dtype_code(weights), _n.ptr(experts), _n.stream()),
+            "om_route_softmax_topk")
+        ctx.save_for_backward(router_logits, experts)
+        ctx.norm_topk_prob = bool(norm_topk_prob)
+        ctx.mark_non_differentiable(experts)
+        return weights, experts
+
+    @staticmethod
+    def backward(ctx, weights_grad, _experts_grad):
+        router_logits, experts = ctx.saved_tensors
+        T, N = router_logits.shape
+        K = experts.shape[1]
+        weights_grad = weights_grad.contiguous()
+        dlogits = torch.empty_like(router_logits)
+        _n.check(_n.lib().om_route_softmax_topk_bwd(
+            _n.ptr(router_logits), _n.dtype_code(router_logits), _n.ptr(experts), _n.ptr(weights_grad),
+            _n.dtype_code(weights_grad), T, N, K, int(ctx.norm_topk_prob), _n.ptr(dlogits),
+            _n.stream()), "om_route_softmax_topk_bwd")
+        return dlogits, None, None, None
+
+
+# ----------------------------------------------------------------------------------------------
+# Index construction (K1 + K2 + K3)
+# ----------------------------------------------------------------------------------------------
+def build_token_permutation(selected_experts, expert_start_idx, expert_end_idx):
+    """Stable counting sort of the (token, k) pairs routed to [expert_start_idx, expert_end_idx).
+
+    Returns device int32 tensors (cum_token_counts [NR+1], cum_expert_counts_ep [T+1],
+    input_indices, output_indices, selected_experts_indices) — the last three sized T*K; only
+    the first cum_token_counts[-1] entries are meaningful.  Same values as the reference's
+    K1 -> cumsum -> K3 sequence (moe.py:499-554).  Nothing is copied to the host."""
+    _n.require_cuda_contiguous(selected_experts)
+    T, K = selected_experts.shape
+    NR = expert_end_idx - expert_start_idx
+    dev = selected_experts.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    cum_token_counts = torch.empty(NR + 1, **i32)
+    cum_expert_counts_ep = torch.empty(T + 1, **i32)
+    input_indices = torch.empty(T * K, **i32)
+    output_indices = torch.empty(T * K, **i32)
+    selected_experts_indices = torch.empty(T * K, **i32)
+    ws_bytes = _n.lib().om_moe_sort_workspace_bytes(T, K, NR)
+    workspace = torch.empty(max(ws_bytes // 4, 1), **i32)
+    _n.check(_n.lib().om_moe_sort(
+        _n.ptr(selected_experts), _n.index_code(selected_experts), T, K, int(expert_start_idx),
+        int(expert_end_idx), _n.ptr(cum_token_counts), _n.ptr(cum_expert_counts_ep),
+        _n.ptr(input_indices), _n.ptr(output_indices), _n.ptr(selected_experts_indices),
+        _n.ptr(workspace), ws_bytes, _n.stream()), "om_moe_sort")
+    return cum_token_counts, cum_expert_counts_ep, input_indices, output_indices, selected_experts_indices
+
+
+# ----------------------------------------------------------------------------------------------
+# Grouped GEMM functions
+# ----------------------------------------------------------------------------------------------
+class GroupedGemmFunction(torch.autograd.Function):
+    """out[s:e] = in[s:e] @ W[g].T per expert segment (reference moe.py:163-215).
+
+    `max_tokens_per_expert` and `use_triton_path` exist for signature parity and are ignored:
+    the kernel sizes its grid from the row count and reads the offsets on the device."""
+
+    @staticmethod
+    def forward(ctx, input, merged_weight, cum_token_counts, max_tokens_per_expert=None,
+                use_triton_path=False):
+        _require_bf16(input, merged_weight)
+        _n.require_cuda_contiguous(input)
+        num_tokens = input.shape[0]
+        num_experts, ofm, ifm = merged_weight.shape
+        cum = _device_counts(cum_token_counts, input.device)
+        output = torch.empty((num_tokens, ofm), dtype=input.dtype, device=input.device)
+        _n.check(_n.lib().om_grouped_gemm_fwd(
+            _n.ptr(input), _n.ptr(merged_weight), _n.ptr(output), _n.ptr(cum), num_tokens,
+            num_experts, ofm, ifm, _expert_stride(merged_weight), _n.stream()), "om_grouped_gemm_fwd")
+        ctx.save_for_backward(input, merged_weight, cum)
+        return output
+
+    @staticmethod
+    def backward(ctx, output_grad):
+        input, merged_weight, cum = ctx.saved_tensors
+        output_grad = output_grad.contiguous()
+        num_experts, ofm, ifm = merged_weight.shape
+        rows = input.shape[0]
+        input_grad = torch.empty_like(input)
+        merged_weight_grad = torch.empty((num_experts, ofm, ifm), dtype=merged_weight.dtype,
+                                         device=merged_weight.device)
+        lib = _n.lib()
+        _n.check(lib.om_grouped_gemm_dgrad(
+            _n.ptr(output_grad), _n.ptr(merged_weight), _n.ptr(input_grad), _n.ptr(cum), rows,
+            num_experts, ofm, ifm, _expert_stride(merged_weight), _n.stream()), "om_grouped_gemm_dgrad")
+        _n.check(lib.om_grouped_gemm_wgrad(
+            _n.ptr(output_grad), _n.ptr(input), _n.ptr(merged_weight_grad), _n.ptr(cum), rows,
+            num_experts, ofm, ifm, 0, _n.stream()), "om_grouped_gemm_wgrad")
+        return input_grad, merged_weight_grad, None, None, None
+
+
+def _merged_mlp_forward(x, w_gate, w_up, w_down, cum_token_counts):
+    """-> (y, cum, g, u, h).  Fused gate+up+SwiGLU launch, then the down projection."""
+    _require_bf16(x, w_gate, w_up, w_down)
+    _n.require_cuda_contiguous(x)
+    rows, H = x.shape
+    G, I, _ = w_gate.shape
+    cum = _device_counts(cum_token_counts, x.device)
+    g = torch.empty((rows, I), dtype=x.dtype, device=x.device)
+    u = torch.empty_like(g)
+    h = torch.empty_like(g)
+    y = torch.empty((rows, H), dtype=x.dtype, device=x.device)
+    lib = _n.lib()
+    sgu = _expert_stride(w_gate)
+    if _expert_stride(w_up) != sgu:
+        raise _n.NativeLibraryError("gate and up expert weights must share one expert pitch")
+    with record_pcl_function("1moeblock--7gmlp_fwd"):
+        _n.check(lib.om_merged_mlp_gate_up_fwd(
+            _n.ptr(x), _n.ptr(w_gate), _n.ptr(w_up), _n.ptr(g), _n.ptr(u), _n.ptr(h), _n.ptr(cum),
+            rows, G, I, H, sgu, _n.stream()), "om_merged_mlp_gate_up_fwd")
+        _n.check(lib.om_grouped_gemm_fwd(
+            _n.ptr(h), _n.ptr(w_down), _n.ptr(y), _n.ptr(cum), rows, G, H, I,
+            _expert_stride(w_down), _n.stream()), "om_grouped_gemm_fwd")
+    return y, cum, g, u, h
+
+
+def _merged_mlp_backward(dy, x, w_gate, w_up, w_down, cum, g, u, h):
+    """-> (dx, dw_gate [G,I,H], dw_up [G,I,H], dw_down [G,H,I]), all freshly allocated."""
+    dy = dy.contiguous()
+    rows, H = x.shape
+    G, I, _ = w_gate.shape
+    lib = _n.lib()
+    st = _n.stream()
+    dg = torch.empty_like(g)
+    du = torch.empty_like(u)
+    dx = torch.empty_like(x)
+    dw_gate = torch.empty((G, I, H), dtype=x.dtype, device=x.device)
+    dw_up = torch.empty((G, I, H), dtype=x.dtype, device=x.device)
+    dw_down = torch.empty((G, H, I), dtype=x.dtype, device=x.device)
+    with record_pcl_function("1moeblock--7gmlp_bwd"):
+        _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(dy), _n.ptr(h), _n.ptr(dw_down), _n.ptr(cum),
+                                           rows, G, H, I, 0, st), "om_grouped_gemm_wgrad(down)")
+        _n.check(lib.om_merged_mlp_down_dgrad(_n.ptr(dy), _n.ptr(w_down), _n.ptr(g), _n.ptr(u),
+                                              _n.ptr(dg), _n.ptr(du), _n.ptr(cum), rows, G, I, H,
+                                              _expert_stride(w_down), st), "om_merged_mlp_down_dgrad")
+        _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(dg), _n.ptr(x), _n.ptr(dw_gate), _n.ptr(cum),
+                                           rows, G, I, H, 0, st), "om_grouped_gemm_wgrad(gate)")
+        _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(du), _n.ptr(x), _n.ptr(dw_up), _n.ptr(cum),
+                                           rows, G, I, H, 0, st), "om_grouped_gemm_wgrad(up)")
+        _n.check(lib.om_merged_mlp_gate_up_dgrad(_n.ptr(dg), _n.ptr(du), _n.ptr(w_gate),
+                                                 _n.ptr(w_up), _n.ptr(dx), _n.ptr(cum), rows, G,
+                                                 I, H, _expert_stride(w_gate), st),
+                 "om_merged_mlp_gate_up_dgrad")
+    return dx, dw_gate, dw_up, dw_down
+
+
+class MergedMLPFunction(torch.autograd.Function):
+    """y = (silu(x Wg^T) * (x Wu^T)) Wd^T per expert segment, with the fused kernels:
+    gate+up+SwiGLU in one launch forward; backward = down dgrad fused with the SwiGLU backward,
+    one dual-operand dgrad for dx, and three weight-gradient GEMMs.
+
+    Same mathematics as the three GroupedGemmFunction calls and two elementwise ops of the
+    reference's MergedMLP.forward (moe.py:396-405) under autograd; g and u are kept in bf16 for
+    the backward like the reference keeps output_gproj / output_uproj."""
+
+    @staticmethod
+    def forward(ctx, x, w_gate, w_up, w_down, cum_token_counts):
+        y, cum, g, u, h = _merged_mlp_forward(x, w_gate, w_up, w_down, cum_token_counts)
+        ctx.save_for_backward(x, w_gate, w_up, w_down, cum, g, u, h)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        dx, dw_gate, dw_up, dw_down = _merged_mlp_backward(dy, *ctx.saved_tensors)
+        return dx, dw_gate, dw_up, dw_down, None
+
+
+class GroupMLPFunction(torch.autograd.Function):
+    """Un-merged layout of the reference (moe.py:43-161): weights arrive as 3*N separate
+    [out, in] tensors (gate_0, up_0, down_0, gate_1, ...).  They must sit at one constant pitch
+    inside a single buffer (true for parameters re-pointed into MixedPrecisionAdamW.flat_param and
+    after pack_expert_weights); the same fused kernels then run on strided views, no copies."""
+
+    @staticmethod
+    def forward(ctx, input, cum_token_counts, use_triton_path, *weight_tuple):
+        N = len(weight_tuple) // 3
+        wg, wu, wd = [_strided_expert_view([weight_tuple[3 * n + j] for n in range(N)])
+                      for j in range(3)]
+        y, cum, g, u, h = _merged_mlp_forward(input, wg, wu, wd, cum_token_counts)
+        ctx.save_for_backward(input, wg, wu, wd, cum, g, u, h)
+        return y
+
+    @staticmethod
+    def backward(ctx, output_grad):
+        dx, dwg, dwu, dwd = _merged_mlp_backward(output_grad, *ctx.saved_tensors)
+        flat = []
+        for n in range(dwg.shape[0]):
+            flat += [dwg[n], dwu[n], dwd[n]]
+        return (dx, None, None, *flat)
+
+
+def _strided_expert_view(weights):
+    """[G, out, in] view over per-expert matrices that lie at a constant pitch in one storage."""
+    w0 = weights[0]
+    o, i = w0.shape
+    G = len(weights)
+    if G == 1:
+        return w0.unsqueeze(0)
+    esz = w0.element_size()
+    pitch_bytes = weights[1].data_ptr() - w0.data_ptr()
+    ok = pitch_bytes > 0 and pitch_bytes % esz == 0 and pitch_bytes >= o * i * esz
+    for n, w in enumerate(weights):
+        ok = ok and w.is_contiguous() and w.shape == w0.shape and w.dtype == w0.dtype \
+            and w.data_ptr() == w0.data_ptr() + n * pitch_bytes \
+            and w.untyped_storage().data_ptr() == w0.untyped_storage().data_ptr()
+    if not ok:
+        raise _n.NativeLibraryError(
+            "per-expert weights must lie at a constant pitch inside one buffer (merge them with "
+            "pack_expert_weights, or build the optimizer first so they alias flat_param)")
+    pitch = pitch_bytes // esz
+    return torch.as_strided(w0, (G, o, i), (pitch, i, 1))
+
+
+def has_constant_pitch(weights):
+    try:
+        _strided_expert_view(weights)
+        return True
+    except _n.NativeLibraryError:
+        return False
+
+
+def pack_expert_weights(experts, names=("gate_proj", "up_proj", "down_proj")):
+    """Make the [out, in] weights of a ModuleList of expert MLPs lie at a constant pitch: where
+    they do not already, re-point them into one buffer per projection (p.data becomes a view,
+    values kept).  Module.to()/.bfloat16() re-allocates parameters one by one, so the blocks call
+    this before they hand the weights to the grouped kernels."""
+    for name in names:
+        ws = [getattr(e, name).weight for e in experts]
+        if has_constant_pitch([w.data for w in ws]):
+            continue
+        buf = torch.stack([w.data for w in ws]).contiguous()
+        for n, w in enumerate(ws):
+            w.data = buf[n]
+
+
+class PrepareInputForGroupGemmFunction(torch.autograd.Function):
+    """K4: ggemm_input = hidden_states[input_indices]; backward sums each token's routed rows in
+    fp32 (reference moe.py:217-282).  The four trailing flags are accepted and ignored."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, input_indices, cum_expert_counts_ep, output_indices,
+                use_ref_path_fwd=False, use_ref_path_bwd=False,
+                use_triton_path_fwd=False, use_triton_path_bwd=False):
+        num_tokens, hidden_dim = hidden_states.shape
+        num_routed_tokens = input_indices.shape[0]
+        with record_pcl_function("1moeblock--6gmlp_input_prep_fwd"):
+            ggemm_input = torch.empty((num_routed_tokens, hidden_dim), dtype=hidden_states.dtype,
+                                      device=hidden_states.device)
+            pcl_xpu_customops.index_gather(hidden_states.contiguous(), input_indices, ggemm_input)
+        ctx.save_for_backward(cum_expert_counts_ep, output_indices)
+        ctx.num_tokens = num_tokens
+        ctx.hidden_dim = hidden_dim
+        return ggemm_input
+
+    @staticmethod
+    def backward(ctx, ggemm_input_grad):
+        cum_expert_counts_ep, output_indices = ctx.saved_tensors
+        with record_pcl_function("1moeblock--6gmlp_input_prep_bwd"):
+            ggemm_input_grad = ggemm_input_grad.contiguous()
+            hidden_states_grad = torch.empty((ctx.num_tokens, ctx.hidden_dim),
+                                             dtype=ggemm_input_grad.dtype,
+                                             device=ggemm_input_grad.device)
+            pcl_xpu_customops.shuffle_sub_matrix_reduce(ggemm_input_grad, cum_expert_counts_ep,
+                                                        output_indices, hidden_states_grad)
+        return hidden_states_grad, None, None, None, None, None, None, None
+
+
+class GroupGemmOutputReductionFunction(torch.autograd.Function):
+    """K6: final[t] = sum_k w[t,k] * ggemm_output[pos(t,k)] in fp32, one rounding; backward gives
+    ggemm_output_grad and routing_weights_grad (reference moe.py:284-377).  The four trailing
+    flags are accepted and ignored.  routing_weights may be fp32 while activations are bf16."""
+
+    @staticmethod
+    def forward(ctx, ggemm_output, routing_weights, cum_expert_counts_ep, selected_experts_indices,
+                input_indices, output_indices,
+                use_ref_path_fwd=False, use_ref_path_bwd=False,
+                use_triton_path_fwd=False, use_triton_path_bwd=False):
+        routing_weights = routing_weights.contiguous()
+        ctx.save_for_backward(ggemm_output, routing_weights, cum_expert_counts_ep,
+                              selected_experts_indices, input_indices, output_indices)
+        num_tokens, _ = routing_weights.shape
+        hidden_dim = ggemm_output.shape[1]
+        with record_pcl_function("1moeblock--8gmlp_output_reduction_fwd"):
+            final_hidden_states = torch.empty((num_tokens, hidden_dim), dtype=ggemm_output.dtype,
+                                              device=ggemm_output.device)
+            pcl_xpu_customops.reduce_ggemm_output(ggemm_output, routing_weights, cum_expert_counts_ep,
+                                                  selected_experts_indices, output_indices,
+                                                  final_hidden_states, False)
+        return final_hidden_states
+
+    @staticmethod
+    def backward(ctx, final_hidden_states_grad):
+        (ggemm_output, routing_weights, cum_expert_counts_ep, selected_experts_indices, input_indices,
+         output_indices) = ctx.saved_tensors
+        final_hidden_states_grad = final_hidden_states_grad.contiguous()
+        ggemm_output_grad = torch.empty_like(ggemm_output)
+        routing_weights_grad = torch.zeros_like(routing_weights)
+        with record_pcl_function("1moeblock--8gmlp_output_reduction_bwd"):
+            pcl_xpu_customops.reduce_ggemm_output_backward(
+                final_hidden_states_grad, ggemm_output, routing_weights, cum_expert_counts_ep,
+                selected_experts_indices, input_indices, output_indices, ggemm_output_grad,
+                routing_weights_grad)
+        return ggemm_output_grad, routing_weights_grad, None, None, None, None, None, None, None, None
+
+
+# ----------------------------------------------------------------------------------------------
+# Modules
+# ----------------------------------------------------------------------------------------------
+class MergedMLP(nn.Module):
+    """All local experts' SwiGLU MLPs as three 3-D parameters (reference moe.py:379-405)."""
+
+    def __init__(self, config):
+        super(MergedMLP, self).__init__()
+        self.config = config
+        self.num_experts_per_rank = config.num_experts // config.expert_parallelism
+        self.gate_proj_merged_weight = torch.nn.Parameter(
+            torch.empty((self.num_experts_per_rank, config.intermediate_size, config.hidden_size)))
+        self.up_proj_merged_weight = torch.nn.Parameter(
+            torch.empty((self.num_experts_per_rank, config.intermediate_size, config.hidden_size)))
+        self.down_proj_merged_weight = torch.nn.Parameter(
+            torch.empty((self.num_experts_per_rank, config.hidden_size, config.intermediate_size)))
+
+    def forward(self, input, cum_token_counts):
+        return MergedMLPFunction.apply(input, self.gate_proj_merged_weight, self.up_proj_merged_weight,
+                                       self.down_proj_merged_weight, cum_token_counts)
+
+
+def expert_computation(hidden_states, routing_weights, selected_experts, expert_start_idx,
+                       expert_end_idx, experts_fn, num_total_experts):
+    """K1..K6 for 2-D hidden_states [T,H]: permute, run `experts_fn(ggemm_input, cum_token_counts)`,
+    combine.  Shared by the OLMoE and DeepSeek-V3 blocks."""
+    T, K = selected_experts.shape
+    with record_pcl_function("1moeblock--3index_calculation"):
+        (cum_token_counts, cum_expert_counts_ep, input_indices, output_indices,
+         selected_experts_indices) = build_token_permutation(selected_experts, expert_start_idx,
+                                                             expert_end_idx)
+    if expert_start_idx == 0 and expert_end_idx == num_total_experts:
+        num_routed_tokens = T * K            # every pair is local: no host read
+    else:
+        num_routed_tokens = int(cum_token_counts[-1].item())   # same host read as moe.py:520
+    input_indices = input_indices[:num_routed_tokens]
+    output_indices = output_indices[:num_routed_tokens]
+    selected_experts_indices = selected_experts_indices[:num_routed_tokens]
+    ggemm_input = PrepareInputForGroupGemmFunction.apply(hidden_states, input_indices,
+                                                         cum_expert_counts_ep, output_indices)
+    ggemm_output = experts_fn(ggemm_input, cum_token_counts)
+    return GroupGemmOutputReductionFunction.apply(ggemm_output, routing_weights, cum_expert_counts_ep,
+                                                  selected_experts_indices, input_indices,
+                                                  output_indices)
+
+
+class FastOlmoeParallelSparseMoeBlock(nn.Module):
+    """Reference moe.py:407-632.  forward(hidden_states [B,S,H]) ->
+    (final_hidden_states [B,S,H], router_logits [B*S,N] or None)."""
+
+    def __init__(self, config, pmap=None):
+        super().__init__()
+        from optimus.models.olmoe.modeling_olmoe import OlmoeParallelMLP
+        self.config = config
+        self.pmap = pmap
+        self.num_experts_per_rank = config.num_experts // config.expert_parallelism
+        self.expert_start_idx = self.pmap.ep_ind * self.num_experts_per_rank
+        self.expert_end_idx = (self.pmap.ep_ind + 1) * self.num_experts_per_rank
+
+        self.hidden_size = config.hidden_size
+        self.intermediate_size = config.intermediate_size
+        self.num_experts = config.num_experts
+        self.num_experts_per_tok = config.num_experts_per_tok
+        self.norm_topk_prob = config.norm_topk_prob
+        self.output_router_logits = config.output_router_logits
+
+        self.gate = nn.Linear(self.hidden_size, self.num_experts, bias=False)
+        if not self.config.use_merged_mlp_in_fast_moe:
+            self.experts = nn.ModuleList([OlmoeParallelMLP(config) for _ in range(self.num_experts_per_rank)])
+        else:
+            self.experts = MergedMLP(config)
+
+        self.use_activation_checkpointing_for_moe = False
+        if config.use_activation_checkpointing:
+            self.use_activation_checkpointing_for_moe = config.activation_checkpointing_level & (1 << 0)
+
+        if getattr(config, "force_uniform_routing", False):
+            raise NotImplementedError("force_uniform_routing is a debug mask of the reference "
+                                      "(moe.py:459-464) and is not part of this build")
+        # fp32 router logits (x.float() @ Wg.float().T) instead of model-dtype logits
+        self.router_logits_fp32 = bool(getattr(config, "router_logits_fp32", False))
+
+    def _experts_fn(self, ggemm_input, cum_token_counts):
+        if isinstance(self.experts, MergedMLP):
+            return self.experts(ggemm_input, cum_token_counts)
+        pack_expert_weights(self.experts)   # no-op once the weights share a buffer
+        mlp_params = []
+        for expert in self.experts:
+            mlp_params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
+        return GroupMLPFunction.apply(ggemm_input, cum_token_counts, False, *mlp_params)
+
+    def forward(self, hidden_states):
+        batch_size, sequence_length, hidden_dim = hidden_states.shape
+        flat = hidden_states.reshape(-1, hidden_dim)
+        if self.router_logits_fp32:
+            router_logits = torch.nn.functional.linear(flat.float(), self.gate.weight.float())
+        else:
+            router_logits = self.gate(flat)
+        routing_weights, selected_experts = SoftmaxTopkRouterFunction.apply(
+            router_logits.contiguous(), self.num_experts_per_tok, self.norm_topk_prob,
+            hidden_states.dtype)
+
+        def expert_computation_block(hidden_states, selected_experts, routing_weights):
+            b, s, h = hidden_states.shape
+            out = expert_computation(hidden_states.reshape(-1, h), routing_weights, selected_experts,
+                                     self.expert_start_idx, self.expert_end_idx, self._experts_fn,
+                                     self.num_experts)
+            return out.reshape(b, s, h)
+
+        args = [hidden_states, selected_experts, routing_weights]
+        if self.use_activation_checkpointing_for_moe:
+            final_hidden_states = torch_activation_checkpoint(expert_computation_block, *args,
+                                                              use_reentrant=False)
+        else:
+            final_hidden_states = expert_computation_block(*args)
+
+        if self.output_router_logits:
+            return final_hidden_states, router_logits
+        return final_hidden_states, None
+
+    def set_parameters_from_full_module(self, module):
+        self.gate.load_state_dict(module.gate.state_dict())
+        with torch.no_grad():
+            for local_expert_idx in range(self.num_experts_per_rank):
+                src = module.experts[self.expert_start_idx + local_expert_idx]
+                if isinstance(self.experts, MergedMLP):
+                    self.experts.gate_proj_merged_weight[local_expert_idx].copy_(src.gate_proj.weight.data)
+                    self.experts.up_proj_merged_weight[local_expert_idx].copy_(src.up_proj.weight.data)
+                    self.experts.down_proj_merged_weight[local_expert_idx].copy_(src.down_proj.weight.data)
+                else:
+                    self.experts[local_expert_idx].load_state_dict(src.state_dict())

@@ -1,0 +1,33 @@
+"""AdamW restatements.  TEST INFRASTRUCTURE ONLY (see oracle/__init__.py).
+
+adamw_step_torch   — the reference's chunked sequence of torch elementwise ops,
+                     optimus/optimizers.py:162-205, on CPU tensors.  This is the "port" that
+                     bench.py times as cpu_baseline for the AdamW workload.
+The scalar C versions (fp32 op-by-op and fp64) are in oracle/adamw_oracle.c via oracle/clib.py.
+"""
+import math
+
+import torch
+
+
+def adamw_step_torch(flat_param, flat_grad, flat_master, flat_exp_avg, flat_exp_avg_sq, step_id,
+                     lr, betas, eps, weight_decay, chunk_size=128 * 1024 * 1024):
+    """In place; step_id is 0-based like MixedPrecisionAdamW.step_id (t = step_id + 1)."""
+    beta1, beta2 = betas
+    size = flat_param.numel()
+    num_chunks = math.ceil(size / chunk_size)                                    # :179-180
+    tensor_list = [flat_param, flat_grad, flat_master, flat_exp_avg, flat_exp_avg_sq]
+    for chunk_id in range(num_chunks):
+        s = chunk_id * chunk_size
+        e = min((chunk_id + 1) * chunk_size, size)
+        data, grad, master, exp_avg, exp_avg_sq = [t[s:e] for t in tensor_list]
+        g32 = grad.to(torch.float32)                                             # :190
+        exp_avg.mul_(beta1).add_(g32, alpha=(1.0 - beta1))                       # :193
+        exp_avg_sq.mul_(beta2).addcmul_(g32, g32, value=1.0 - beta2)             # :194
+        exp_avg_hat = exp_avg / (1.0 - math.pow(beta1, (step_id + 1)))           # :195
+        exp_avg_sq_hat = exp_avg_sq / (1.0 - math.pow(beta2, (step_id + 1)))     # :196
+        denom = exp_avg_sq_hat.sqrt().add_(eps)                                  # :197
+        master.addcdiv_(exp_avg_hat, denom, value=-lr)                           # :198
+        if weight_decay > 0.0:
+            master.add_(master, alpha=(-lr * weight_decay))                      # :202
+        data.copy_(master.to(data.dtype))                                        # :205

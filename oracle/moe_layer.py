@@ -1,0 +1,141 @@
+"""Whole-layer restatements in PyTorch-CPU.  TEST INFRASTRUCTURE ONLY (see oracle/__init__.py).
+
+* expert_mlp / olmoe_slow_block — optimus/models/olmoe/modeling_olmoe.py:239-251, :282-354
+  (the reference's per-expert one-hot / where / index_add_ loop; backward by autograd).
+* dsv3_moe_block                — optimus/models/deepseek_v3/modeling_deepseek_v3.py:221-275.
+* fast_block_restatement        — optimus/models/common/moe.py:454-621 with the K1..K6
+  operators taken from the C restatement of the SYCL kernels (oracle/clib.py) and the expert
+  GEMMs as per-expert torch.matmul on slices (moe.py:174-178).
+* dense_formula                 — the textbook statement out[t] = sum_k w[t,k] MLP_{e[t,k]}(x[t]),
+  evaluated token by token; used on tiny shapes to pin the two loops above.
+
+All functions take plain tensors (no nn.Module) so the tests read as data in / data out.
+"""
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+from . import clib
+from . import routing
+
+
+def expert_mlp(x, w_gate, w_up, w_down):
+    """down(silu(gate(x)) * up(x)); weights are [out, in] like nn.Linear (modeling_olmoe.py:249-251)."""
+    return F.linear(F.silu(F.linear(x, w_gate)) * F.linear(x, w_up), w_down)
+
+
+def olmoe_slow_block(hidden_states, gate_weight, w_gate, w_up, w_down, top_k, norm_topk_prob,
+                     expert_start_idx=0, router_logits=None):
+    """modeling_olmoe.py:282-354 with expert_parallelism == 1 semantics for the window.
+
+    hidden_states [T,H]; gate_weight [N,H]; w_gate/w_up [NR,I,H]; w_down [NR,H,I].
+    Accumulates in hidden_states.dtype via index_add_ in expert order, like the reference.
+    Returns (final_hidden_states [T,H], router_logits [T,N]).
+    """
+    T, H = hidden_states.shape
+    N = gate_weight.shape[0]
+    NR = w_gate.shape[0]
+    if router_logits is None:
+        router_logits = F.linear(hidden_states, gate_weight)                       # :284
+    routing_weights, selected_experts, _ = routing.olmoe_router(
+        router_logits, top_k, norm_topk_prob, hidden_states.dtype)                 # :295-299
+    final = torch.zeros((T, H), dtype=hidden_states.dtype)                         # :311-313
+    expert_mask = F.one_hot(selected_experts, num_classes=N).permute(2, 1, 0)      # :316
+    for local_expert_idx in range(NR):                                             # :322
+        expert_idx = expert_start_idx + local_expert_idx
+        idx, top_x = torch.where(expert_mask[expert_idx])                          # :325
+        current_state = hidden_states[None, top_x].reshape(-1, H)                  # :330
+        current = expert_mlp(current_state, w_gate[local_expert_idx], w_up[local_expert_idx],
+                             w_down[local_expert_idx]) * routing_weights[top_x, idx, None]  # :331
+        final.index_add_(0, top_x, current)                                        # :336
+    return final, router_logits
+
+
+def dsv3_moe_block(hidden_states, router_weight, bias, w_gate, w_up, w_down,
+                   ws_gate, ws_up, ws_down, n_group, topk_group, top_k, norm_topk_prob,
+                   routed_scaling_factor, expert_start_idx=0):
+    """modeling_deepseek_v3.py:221-275 for one rank's window of routed experts + shared expert.
+
+    The routed part accumulates in the routing-weight dtype (fp32) and is cast once (:222, :244).
+    """
+    T, H = hidden_states.shape
+    N = router_weight.shape[0]
+    NR = w_gate.shape[0]
+    topk_indices, topk_weights, _ = routing.dsv3_router(
+        hidden_states, router_weight, bias, n_group, topk_group, top_k, norm_topk_prob,
+        routed_scaling_factor)
+    final = torch.zeros((T, H), dtype=topk_weights.dtype)                          # :222
+    expert_mask = F.one_hot(topk_indices, num_classes=N).permute(2, 0, 1)          # :224-225
+    for local_expert_idx in range(NR):
+        expert_idx = expert_start_idx + local_expert_idx
+        token_indices, weight_indices = torch.where(expert_mask[expert_idx])       # :232
+        if token_indices.numel() > 0:
+            expert_weights = topk_weights[token_indices, weight_indices]
+            expert_output = expert_mlp(hidden_states[token_indices], w_gate[local_expert_idx],
+                                       w_up[local_expert_idx], w_down[local_expert_idx])
+            final.index_add_(0, token_indices, expert_output * expert_weights.unsqueeze(-1))  # :239
+    out = final.type(hidden_states.dtype)                                          # :244
+    out = out + expert_mlp(hidden_states, ws_gate, ws_up, ws_down)                 # :265
+    return out, topk_indices, topk_weights
+
+
+def dense_formula(hidden_states, routing_weights, selected_experts, w_gate, w_up, w_down,
+                  expert_start_idx=0):
+    """out[t] = sum over k with a local expert of w[t,k] * MLP_{e[t,k]}(x[t]); token-by-token loop."""
+    T, H = hidden_states.shape
+    NR = w_gate.shape[0]
+    rows = []
+    for t in range(T):
+        acc = torch.zeros(H, dtype=hidden_states.dtype)
+        for k in range(selected_experts.shape[1]):
+            ln = int(selected_experts[t, k]) - expert_start_idx
+            if 0 <= ln < NR:
+                acc = acc + routing_weights[t, k] * expert_mlp(hidden_states[t:t + 1], w_gate[ln],
+                                                                w_up[ln], w_down[ln])[0]
+        rows.append(acc)
+    return torch.stack(rows)
+
+
+def _np(t):
+    """torch tensor -> numpy (bf16 as raw uint16 bits)."""
+    if t.dtype == torch.bfloat16:
+        return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    return t.contiguous().numpy()
+
+
+def _pt(a, dtype):
+    if dtype == torch.bfloat16:
+        return torch.from_numpy(a.view(np.int16)).view(torch.bfloat16)
+    return torch.from_numpy(a)
+
+
+def fast_block_restatement(hidden_states, routing_weights, selected_experts, w_gate, w_up, w_down,
+                           expert_start_idx=0):
+    """Forward of expert_computation_block (moe.py:473-610) for EP == 1 style windows.
+
+    hidden_states [T,H] fp32 or bf16; selected_experts [T,K] int64; merged weights [NR,*,*].
+    K1..K3, K4f and K6f come from the C restatement of the SYCL kernels; the grouped GEMM is
+    the reference's loop of per-expert matmuls (moe.py:174-178) and SwiGLU the two torch ops of
+    MergedMLP.forward (moe.py:401-402).  Returns (final [T,H], dict of intermediates).
+    """
+    dt = hidden_states.dtype
+    NR = w_gate.shape[0]
+    idx = clib.index_construction(selected_experts.numpy(), NR, expert_start_idx,
+                                  expert_start_idx + NR)
+    ggemm_input = _pt(clib.index_gather(_np(hidden_states), idx["input_indices"]), dt)
+    cum = idx["cum_token_counts"]
+    g = torch.empty((ggemm_input.shape[0], w_gate.shape[1]), dtype=dt)
+    u = torch.empty_like(g)
+    for n in range(NR):
+        s, e = int(cum[n]), int(cum[n + 1])
+        torch.matmul(ggemm_input[s:e], w_gate[n].t(), out=g[s:e])
+        torch.matmul(ggemm_input[s:e], w_up[n].t(), out=u[s:e])
+    h = F.silu(g) * u
+    y = torch.empty((ggemm_input.shape[0], w_down.shape[1]), dtype=dt)
+    for n in range(NR):
+        s, e = int(cum[n]), int(cum[n + 1])
+        torch.matmul(h[s:e], w_down[n].t(), out=y[s:e])
+    final = _pt(clib.reduce_ggemm_output(_np(y), _np(routing_weights), idx["cum_expert_counts_ep"],
+                                         idx["selected_experts_indices"], idx["output_indices"]), dt)
+    idx.update(ggemm_input=ggemm_input, g=g, u=u, h=h, ggemm_output=y)
+    return final, idx

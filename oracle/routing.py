@@ -1,0 +1,73 @@
+"""Router restatements in PyTorch-CPU.  TEST INFRASTRUCTURE ONLY (see oracle/__init__.py).
+
+* olmoe_router        — optimus/models/common/moe.py:467-471
+                        (= optimus/models/olmoe/modeling_olmoe.py:295-299)
+* dsv3_topk_indices   — optimus/models/deepseek_v3/modeling_deepseek_v3.py:164-180
+* dsv3_router         — optimus/models/deepseek_v3/modeling_deepseek_v3.py:182-192
+
+Tie-break.  The reference calls torch.topk, whose order among equal values is an
+implementation property.  The oracle fixes it: among equal scores the lower expert
+index comes first (a stable descending sort).  On rows without ties this is exactly
+torch.topk(sorted=True); tests/test_oracle_routing.py checks that against the library
+call.  For the DeepSeek router the reference asks for sorted=False, so the order of a
+token's K experts is unspecified there; the oracle returns them in descending
+score-for-choice order and parity on that path is per-token *sets* plus weights.
+"""
+import torch
+
+
+def _topk_stable(values, k):
+    """Top-k along the last dim, descending, lower index first among equals."""
+    s = torch.sort(values, dim=-1, descending=True, stable=True)
+    return s.values[..., :k].contiguous(), s.indices[..., :k].contiguous()
+
+
+def olmoe_router(router_logits, top_k, norm_topk_prob, out_dtype):
+    """-> (routing_weights [T,K] out_dtype, selected_experts [T,K] int64, probs [T,N] fp32)."""
+    probs = torch.softmax(router_logits, dim=1, dtype=torch.float)       # moe.py:467
+    routing_weights, selected_experts = _topk_stable(probs, top_k)       # moe.py:468
+    if norm_topk_prob:
+        routing_weights = routing_weights / routing_weights.sum(dim=-1, keepdim=True)  # :469-470
+    return routing_weights.to(out_dtype), selected_experts, probs        # :471
+
+
+def min_topk_gap_ulps(scores, top_k):
+    """Smallest gap, in units of fp32 ulp of the larger neighbour, between adjacent entries
+    of each row's top-(K+1) scores.  Fixtures are valid for bit-exact index parity when this
+    exceeds a few ulp: a last-ulp difference between two exp() implementations cannot then
+    reorder a row."""
+    k1 = min(top_k + 1, scores.shape[-1])
+    top = torch.sort(scores.float(), dim=-1, descending=True).values[..., :k1]
+    gap = top[..., :-1] - top[..., 1:]
+    ulp = torch.abs(top[..., :-1]) * (2.0 ** -23)
+    return float((gap / ulp.clamp_min(1e-45)).min())
+
+
+def dsv3_topk_indices(scores, bias, n_group, topk_group, top_k):
+    """Group-limited selection, modeling_deepseek_v3.py:164-180 (sorted=False there)."""
+    T, N = scores.shape
+    scores_for_choice = scores.view(-1, N) + bias.unsqueeze(0)                        # :164
+    per_group = scores_for_choice.view(-1, n_group, N // n_group)
+    group_scores = _topk_stable(per_group, 2)[0].sum(dim=-1)                          # :165-169
+    group_idx = _topk_stable(group_scores, topk_group)[1]                             # :170
+    group_mask = torch.zeros_like(group_scores)
+    group_mask.scatter_(1, group_idx, 1)                                              # :171-172
+    score_mask = (group_mask.unsqueeze(-1).expand(-1, n_group, N // n_group).reshape(-1, N))
+    scores_for_choice = scores_for_choice.masked_fill(~score_mask.bool(), 0.0)        # :178
+    return _topk_stable(scores_for_choice, top_k)[1], scores_for_choice               # :179
+
+
+def dsv3_router(hidden_states, weight, bias, n_group, topk_group, top_k, norm_topk_prob,
+                routed_scaling_factor):
+    """-> (topk_indices [T,K] int64, topk_weights [T,K] fp32, router_logits fp32)."""
+    x = hidden_states.reshape(-1, hidden_states.shape[-1])
+    router_logits = torch.nn.functional.linear(x.type(torch.float32), weight.type(torch.float32))
+    scores = router_logits.sigmoid()                                                  # :185
+    with torch.no_grad():
+        topk_indices, _ = dsv3_topk_indices(scores, bias.float(), n_group, topk_group, top_k)
+    topk_weights = scores.gather(1, topk_indices)                                     # :187
+    if norm_topk_prob:
+        denominator = topk_weights.sum(dim=-1, keepdim=True) + 1e-20                  # :189
+        topk_weights = topk_weights / denominator
+    topk_weights = topk_weights * routed_scaling_factor                               # :191
+    return topk_indices, topk_weights, router_logits

@@ -1,0 +1,104 @@
+"""Grouped expert GEMMs through optimus.models.common.moe (-> C-ABI om_grouped_gemm_*,
+om_merged_mlp_*) against per-expert torch.matmul in fp32 on the same bf16 inputs — the special
+case the reference itself uses as its check (optimus/kernels/grouped_linear_forward.py:104-112,
+moe.py:174-178).  Bar: outputs are bf16 roundings of fp32-accumulated sums, so the error is at
+most a bf16 half-ulp of the result plus fp32 summation-order noise: max-abs <= 2e-2 and mean-rel
+<= 1e-3 (the layer tolerance), checked per product."""
+import numpy as np
+import pytest
+import torch
+
+from util import max_abs, mean_rel
+
+pytestmark = pytest.mark.gpu
+
+
+def _counts(kind, G, rows, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "uniform":
+        c = torch.full((G,), rows // G)
+        c[: rows - int(c.sum())] += 1
+    elif kind == "ragged":
+        p = torch.rand(G, generator=g) ** 3
+        c = torch.floor(p / p.sum() * rows).long()
+        c[0] += rows - int(c.sum())
+    elif kind == "empties":
+        c = torch.zeros(G, dtype=torch.long)
+        hot = torch.randperm(G, generator=g)[: max(1, G // 4)]
+        c[hot] = rows // len(hot)
+        c[hot[0]] += rows - int(c.sum())
+    cum = torch.zeros(G + 1, dtype=torch.int32)
+    cum[1:] = torch.cumsum(c, 0)
+    return cum
+
+
+def _ref_fwd(x, w, cum):
+    out = torch.zeros(x.shape[0], w.shape[1])
+    for g in range(w.shape[0]):
+        s, e = int(cum[g]), int(cum[g + 1])
+        out[s:e] = x[s:e].float() @ w[g].float().t()
+    return out
+
+
+CASES = [("uniform", 4, 512, 256, 128), ("ragged", 8, 1000, 256, 512), ("empties", 16, 777, 128, 256),
+         ("ragged", 64, 4096, 1024, 2048), ("uniform", 1, 300, 256, 256), ("ragged", 3, 5, 128, 128)]
+
+
+@pytest.mark.parametrize("kind,G,rows,N,K", CASES)
+def test_grouped_gemm_fwd_dgrad_wgrad(cuda, kind, G, rows, N, K):
+    from optimus.models.common.moe import GroupedGemmFunction
+    g = torch.Generator().manual_seed(rows)
+    x = torch.randn(rows, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(G, N, K, generator=g) * 0.05).to(torch.bfloat16)
+    dout = torch.randn(rows, N, generator=g).to(torch.bfloat16)
+    cum = _counts(kind, G, rows)
+    xd = x.to(cuda).requires_grad_(True)
+    wd = w.to(cuda).requires_grad_(True)
+    # the reference passes a CPU int32 tensor of offsets and max_tokens_per_expert (moe.py:397-398)
+    out = GroupedGemmFunction.apply(xd, wd, cum, int((cum[1:] - cum[:-1]).max()), False)
+    out.backward(dout.to(cuda))
+    ref = _ref_fwd(x, w, cum)
+    assert max_abs(out.float().cpu(), ref) <= 2e-2 * max(1.0, float(ref.abs().max()))
+    assert mean_rel(out.float().cpu(), ref) <= 4e-3      # one bf16 rounding: ~2^-9 relative
+    dx_ref = torch.zeros(rows, K); dw_ref = torch.zeros(G, N, K)
+    for e in range(G):
+        s, t = int(cum[e]), int(cum[e + 1])
+        dx_ref[s:t] = dout[s:t].float() @ w[e].float()
+        dw_ref[e] = dout[s:t].float().t() @ x[s:t].float()
+    assert mean_rel(xd.grad.float().cpu(), dx_ref) <= 4e-3
+    assert mean_rel(wd.grad.float().cpu(), dw_ref) <= 4e-3
+    assert max_abs(wd.grad.float().cpu(), dw_ref) <= 1e-2 * max(1.0, float(dw_ref.abs().max()))
+    # experts without rows get exactly zero weight gradient
+    empty = (cum[1:] == cum[:-1])
+    if empty.any():
+        assert float(wd.grad[empty.to(cuda)].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("kind,G,rows,I,H", [("uniform", 4, 512, 128, 256), ("ragged", 8, 1500, 512, 256),
+                                            ("empties", 64, 4096, 1024, 2048), ("ragged", 2, 7, 128, 128)])
+def test_merged_mlp_fused(cuda, kind, G, rows, I, H):
+    """MergedMLP (fused gate+up+SwiGLU, fused down-dgrad+SwiGLU-backward, dual dgrad) against the
+    fp32 composition silu(x Wg^T) * (x Wu^T) Wd^T under autograd."""
+    from optimus.models.common.moe import MergedMLPFunction
+    g = torch.Generator().manual_seed(rows + 1)
+    x = torch.randn(rows, H, generator=g).to(torch.bfloat16)
+    wg = (torch.randn(G, I, H, generator=g) * 0.05).to(torch.bfloat16)
+    wu = (torch.randn(G, I, H, generator=g) * 0.05).to(torch.bfloat16)
+    wd = (torch.randn(G, H, I, generator=g) * 0.05).to(torch.bfloat16)
+    dy = torch.randn(rows, H, generator=g).to(torch.bfloat16)
+    cum = _counts(kind, G, rows)
+    dev = [t.to(cuda).requires_grad_(True) for t in (x, wg, wu, wd)]
+    y = MergedMLPFunction.apply(*dev, cum.to(cuda))
+    y.backward(dy.to(cuda))
+    ref = [t.float().requires_grad_(True) for t in (x, wg, wu, wd)]
+    outs = []
+    for e in range(G):
+        s, t = int(cum[e]), int(cum[e + 1])
+        xe = ref[0][s:t]
+        outs.append((torch.nn.functional.silu(xe @ ref[1][e].t()) * (xe @ ref[2][e].t())) @ ref[3][e].t())
+    yr = torch.cat(outs)
+    yr.backward(dy.float())
+    assert mean_rel(y.float().cpu(), yr.detach()) <= 6e-3
+    assert max_abs(y.float().cpu(), yr.detach()) <= 2e-2 * max(1.0, float(yr.abs().max()))
+    for name, a, b in zip(("dx", "dwg", "dwu", "dwd"), dev, ref):
+        assert mean_rel(a.grad.float().cpu(), b.grad) <= 1e-2, name
