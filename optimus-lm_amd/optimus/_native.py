@@ -71,9 +71,40 @@ SIGNATURES = {
 
 _lib = None
 
+# Optional per-launch timing: when set to a list, every call of a kernel-launching entry point
+# appends (name, start_event, end_event) recorded on the current stream.  Used by bench.py to get
+# kernel durations from HIP events inside the timed region; None (the default) costs one test.
+launch_log = None
+_UNTIMED = {"om_version", "om_arch", "om_strerror", "om_moe_sort_workspace_bytes"}
+
 
 class NativeLibraryError(RuntimeError):
     pass
+
+
+class _Library:
+    """The loaded C-ABI functions as attributes (om_adamw_step, ...)."""
+
+    def __init__(self, handle):
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+            setattr(self, name, fn if name in _UNTIMED else self._maybe_timed(name, fn))
+
+    @staticmethod
+    def _maybe_timed(name, fn):
+        def call(*args):
+            if launch_log is None:
+                return fn(*args)
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+            rc = fn(*args)
+            b.record()
+            launch_log.append((name, a, b))
+            return rc
+        return call
 
 
 def lib():
@@ -84,12 +115,7 @@ def lib():
             raise NativeLibraryError(
                 f"{LIB_PATH} not found: build it with `python optimus-lm_amd/build.py` "
                 "(there is no non-HIP fallback)")
-        handle = ctypes.CDLL(LIB_PATH)
-        for name, (res, args) in SIGNATURES.items():
-            fn = getattr(handle, name)
-            fn.restype = res
-            fn.argtypes = args
-        _lib = handle
+        _lib = _Library(ctypes.CDLL(LIB_PATH))
     return _lib
 
 

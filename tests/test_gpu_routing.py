@@ -51,6 +51,7 @@ def test_softmax_topk_bf16_logits_and_ties(cuda):
     g = torch.Generator().manual_seed(0)
     logits = torch.randn(4096, 64, generator=g).to(torch.bfloat16)
     logits[:64] = 0.0            # all equal: experts 0..K-1 in order
+    logits[64:128] = logits[64:128].clamp(max=2.0)
     logits[64:128, 10:20] = 3.0  # ten-way tie above the rest: 10..17
     w, e = F.apply(logits.to(cuda), 8, False, torch.float32)
     e = e.cpu()
