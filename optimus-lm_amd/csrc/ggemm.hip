@@ -3,22 +3,28 @@
 // One kernel template covers every product of the merged MLP.  An output tile BM x BN is
 // computed by WAVES_M x WAVES_N wavefronts; each wavefront owns a (BM/WAVES_M) x (BN/WAVES_N)
 // sub-tile as a grid of 32x32 MFMA accumulators.  Operands are staged through LDS in steps of
-// 64 along the contraction index c, double buffered, one barrier per step.
+// 64 along the contraction index c with direct global->LDS loads (global_load_lds_dwordx4: no
+// register staging, no ds_write), two LDS stages, one barrier per step: the loads of step s+1
+// are in flight while step s is multiplied.
 //
 // An operand is either
 //   CONTIG  — stored [row][c] with c contiguous (activations in fwd/dgrad, weights in fwd):
 //             LDS keeps 128-byte rows with the 16-byte chunks XOR-permuted per row; a fragment
 //             is one ds_read_b128 per lane;
 //   STRIDED — stored [c][row] with row contiguous (weights in dgrad, both operands in wgrad):
-//             LDS keeps the tile as it lies in memory; fragments come from the gfx950
-//             transposing LDS read (ds_read_b64_tr_b16), two per lane.
-// The per-lane order of the 8 contraction indices is the same for both kinds, so they can be
-// mixed in one MFMA.
+//             LDS keeps the tile as it lies in memory (chunks XOR-permuted per c-row); fragments
+//             come from the gfx950 transposing LDS read (ds_read_b64_tr_b16), two per lane.
+// A direct load writes LDS at (wave-uniform base + lane*16), so the permutation is applied by
+// choosing which global chunk each lane fetches.  The per-lane order of the 8 contraction
+// indices is the same for both kinds, so they can be mixed in one MFMA.
 //
 // Variable rows per expert: the M extent of fwd/dgrad is cut into tiles per expert; a block finds
 // its (expert, row block) from the device-resident cum_token_counts with a wavefront scan, so no
 // host copy of the counts and no max-rows-per-expert is needed.  In wgrad the rows are the
-// contraction range of expert g and rows past its end are zero-filled.
+// contraction range of expert g; rows past its end are zero-filled in LDS.
+//
+// Block order: consecutive block ids go to different XCDs (8 per chip, each with its own L2), so
+// block ids are remapped to give every XCD a contiguous run of tiles, which share operand tiles.
 #include "common.h"
 
 namespace {
@@ -32,6 +38,7 @@ enum {
 };
 
 constexpr int BK = 64;  // contraction step, elements
+constexpr int NUM_XCD = 8;
 
 struct GemmParams {
     // operands; for the two-phase products (gate+up) index 1 is the second pair
@@ -53,23 +60,27 @@ struct GemmParams {
     int m_tiles_max;            // fwd/dgrad: upper bound on row tiles
 };
 
-__device__ __forceinline__ int swz(int row) { return (row + (row >> 3)) & 7; }
+typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_ptr;
+typedef __attribute__((address_space(3))) void *lds_void_ptr;
+typedef const __attribute__((address_space(1))) void *glb_void_ptr;
 
-// LDS byte offset of 16-byte chunk `ch` of row `row` in a CONTIG tile.
+// 16 bytes global -> LDS; LDS address = lds_base (wave-uniform) + lane*16.
+__device__ __forceinline__ void load16_to_lds(const void *gptr, char *lds_base) {
+    __builtin_amdgcn_global_load_lds((glb_void_ptr)gptr, (lds_void_ptr)lds_base, 16, 0, 0);
+}
+
+// ---- CONTIG tile: R rows x 64 c; 128-byte rows; chunk position = chunk ^ swz(row) ----------
+__device__ __forceinline__ int swz(int row) { return ((row & 31) + ((row & 31) >> 3)) & 7; }  // period 32
 __device__ __forceinline__ int contig_off(int row, int ch) { return row * 128 + ((ch ^ swz(row)) << 4); }
 
-template <int R> struct StridedTile {
-    static constexpr int PITCH = R * 2 + 64;  // bytes per c-row; +64 spreads rows over the banks
-    static constexpr int BYTES = BK * PITCH;
-};
-template <int R> struct ContigTile {
-    static constexpr int BYTES = R * 128;
-};
-template <int KIND, int R> struct TileBytes {
-    static constexpr int value = KIND == CONTIG ? ContigTile<R>::BYTES : StridedTile<R>::BYTES;
-};
+// ---- STRIDED tile: 64 c-rows x R rows-of-the-operand; R*2-byte c-rows; chunk position =
+//      chunk ^ ((crow & 3) << 2): the four c-rows a transposing read touches land in four
+//      different 64-byte bank windows -------------------------------------------------------
+template <int R> __device__ __forceinline__ int strided_off(int crow, int ch) {
+    return crow * (R * 2) + ((ch ^ ((crow & 3) << 2)) << 4);
+}
 
-typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_ptr;
+template <int KIND, int R> struct TileBytes { static constexpr int value = R * 128; };  // both kinds
 
 __device__ __forceinline__ bf16x8 lds_read_frag_contig(const char *tile, int row, int ch) {
     const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + contig_off(row, ch));
@@ -84,9 +95,11 @@ __device__ __forceinline__ bf16x8 lds_read_frag_strided(const char *tile, int c0
     const int r = i >> 2, q = i & 3;
     const int mb = ((lane >> 4) & 1) * 16;
     const int g2 = lane >> 5;
-    const char *p = tile + (c0 + 8 * g2 + r) * StridedTile<R>::PITCH + (m0 + mb + 4 * q) * 2;
+    const int m = m0 + mb + 4 * q;
+    const int cr = c0 + 8 * g2 + r;  // (cr & 3) == (cr + 4) & 3
+    const char *p = tile + strided_off<R>(cr, m >> 3) + (m & 7) * 2;
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * StridedTile<R>::PITCH));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * R * 2));
     typedef __attribute__((ext_vector_type(8))) short s16x8;
     s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(bf16x8, v);
@@ -140,15 +153,28 @@ __device__ __forceinline__ bool find_tile(const int32_t *cum, int n_experts, int
     return false;
 }
 
+// Give every XCD a contiguous run of logical tiles (hardware sends block b to XCD b % 8).
+__device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
+    const int per = nblocks / NUM_XCD;       // blocks in the evenly divisible part
+    const int body = per * NUM_XCD;
+    if (bid >= body) return bid;             // tail keeps its order
+    return (bid % NUM_XCD) * per + bid / NUM_XCD;
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const GemmParams p) {
-    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
     constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 accumulators per wavefront
     constexpr int A_BYTES = TileBytes<AKIND, BM>::value;
     constexpr int B_BYTES = TileBytes<BKIND, BN>::value;
-    constexpr int STAGE = A_BYTES + B_BYTES;
-    extern __shared__ __attribute__((aligned(16))) char smem[];  // 2 stages
+    constexpr int A_LOADS = BM / 8 / NW;                 // direct loads per wavefront per step
+    constexpr int B_LOADS = BN / 8 / NW;
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/wave mismatch");
+    // two statically distinct stages: the compiler can then tell that a fragment read of one
+    // stage does not depend on the loads in flight to the other
+    __shared__ __attribute__((aligned(1024))) char stage0[A_BYTES + B_BYTES];
+    __shared__ __attribute__((aligned(1024))) char stage1[A_BYTES + B_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -158,10 +184,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // ---- which tile ---------------------------------------------------------------------
     int expert, row_begin, row_end;  // fwd/dgrad: rows of this tile's expert segment
     int n0;                          // first output column (LDS B row 0)
-    int64_t c_begin, c_len;          // contraction range
+    int c_begin, c_len;              // contraction range
     if (EPI == EPI_WGRAD) {
         // grid: x = (N/BM) * (K/BN) tiles of dW[g], y = expert
-        const int tiles_n = p.n_cols / BN;  // n_cols = K_orig (columns of dW), rows of dW = p.kc
+        const int tiles_n = p.n_cols / BN;
         expert = blockIdx.y;
         const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
         row_begin = tm * BM;  // row of dW
@@ -172,100 +198,118 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     } else {
         constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
         const int tiles_n = p.n_cols / BN_OUT;
-        const int tile_m = blockIdx.x / tiles_n;
-        const int tile_n = blockIdx.x % tiles_n;
+        const int logical = xcd_remap(blockIdx.x, gridDim.x);
+        const int tile_m = logical / tiles_n;
+        const int tile_n = logical % tiles_n;
         if (!find_tile<BM>(p.cum, p.n_experts, tile_m, lane, expert, row_begin, row_end)) return;
         n0 = tile_n * BN_OUT;
         c_begin = 0;
         c_len = p.kc;
     }
-    const int phases = p.phases;
-    const int steps_per_phase = static_cast<int>((c_len + BK - 1) / BK);
-    const int total_steps = steps_per_phase * phases;
+    const int steps_per_phase = (c_len + BK - 1) / BK;
+    const int total_steps = steps_per_phase * p.phases;
 
-    // ---- global -> register staging ---------------------------------------------------------
-    constexpr int A_CHUNKS = BM * 8 / NT;  // 16-byte chunks per thread per step
-    constexpr int B_CHUNKS = BN * 8 / NT;
-    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile/thread mismatch");
-    u32x4 ra[A_CHUNKS], rb[B_CHUNKS];
-
-    auto load_tiles = [&](int step) {
-        const int ph = step / steps_per_phase;
-        const int64_t c0 = static_cast<int64_t>(step - ph * steps_per_phase) * BK;
-        const uint16_t *Ap = p.A[ph];
-        const uint16_t *Bp = p.B[ph];
+    // ---- per-lane source offsets of the direct loads (elements, without the c0 term) ------------
+    // CONTIG : lane -> (row = group*8 + lane/8, chunk = (lane%8) ^ swz(row))
+    // STRIDED: lane -> (crow = group*(64/CPR) + lane/CPR, chunk = (lane%CPR) ^ ((crow&3)<<2))
+    int a_off[A_LOADS], b_off[B_LOADS];  // the host checks that every operand spans < 2^31 elements
+    int a_crow[A_LOADS];  // STRIDED A in wgrad: c-row of the lane's slot (for the zero fill)
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; i++) {
-            const int q = tid + i * NT;
-            if (AKIND == CONTIG) {
-                const int row = q >> 3, ch = q & 7;
-                int64_t m = static_cast<int64_t>(row_begin) + row;
-                if (m >= row_end) m = row_end - 1;  // rows past the segment: valid memory, result unused
-                ra[i] = *reinterpret_cast<const u32x4 *>(Ap + m * p.lda + c0 + ch * 8);
+    for (int i = 0; i < A_LOADS; i++) {
+        const int grp = wave * A_LOADS + i;
+        if (AKIND == CONTIG) {
+            const int row = grp * 8 + (lane >> 3);
+            const int ch = (lane & 7) ^ swz(row);
+            int64_t m = static_cast<int64_t>(row_begin) + row;
+            if (m >= row_end) m = row_end - 1;  // rows past the segment: valid memory, result unused
+            a_off[i] = static_cast<int>(m * p.lda + ch * 8);
+            a_crow[i] = 0;
+        } else {
+            constexpr int CPR = BM / 8;
+            const int crow = grp * (64 / CPR) + lane / CPR;
+            const int ch = (lane % CPR) ^ ((crow & 3) << 2);
+            a_off[i] = row_begin + ch * 8;  // + (c_begin + c) * lda per step
+            a_crow[i] = crow;
+        }
+    }
+    int b_crow[B_LOADS];
+    bool b_up[B_LOADS];  // EPI_SWIGLU: this LDS row comes from the up matrix
+#pragma unroll
+    for (int i = 0; i < B_LOADS; i++) {
+        const int grp = wave * B_LOADS + i;
+        if (BKIND == CONTIG) {
+            const int row = grp * 8 + (lane >> 3);
+            const int ch = (lane & 7) ^ swz(row);
+            if (EPI == EPI_SWIGLU) {
+                // LDS rows alternate 32 gate rows / 32 up rows; the up matrix is B[1]
+                const int blk = row >> 5;
+                const int64_t n = n0 + (blk >> 1) * 32 + (row & 31);
+                b_off[i] = static_cast<int>(expert * p.strideB + n * p.ldb + ch * 8);
+                b_up[i] = blk & 1;
             } else {
-                constexpr int CPR = BM / 8;
-                const int crow = q / CPR, ch = q % CPR;
-                const int64_t c = c0 + crow;
-                if (c < c_len)
-                    ra[i] = *reinterpret_cast<const u32x4 *>(Ap + (c_begin + c) * p.lda + row_begin + ch * 8);
-                else
-                    ra[i] = u32x4{0, 0, 0, 0};
+                b_off[i] = static_cast<int>(expert * p.strideB + static_cast<int64_t>(n0 + row) * p.ldb + ch * 8);
             }
+            b_crow[i] = 0;
+            if (EPI != EPI_SWIGLU) b_up[i] = false;
+        } else {
+            b_up[i] = false;
+            constexpr int CPR = BN / 8;
+            const int crow = grp * (64 / CPR) + lane / CPR;
+            const int ch = (lane % CPR) ^ ((crow & 3) << 2);
+            b_off[i] = static_cast<int>((EPI == EPI_WGRAD ? 0 : expert * p.strideB) + n0 + ch * 8);
+            b_crow[i] = crow;
+        }
+    }
+
+    // Loads of contraction step `step` into `stage`.  Steps past the end (the loop always works on
+    // pairs of steps) re-read the last valid slice; their data is never multiplied, or is zeroed.
+    const int lda32 = static_cast<int>(p.lda), ldb32 = static_cast<int>(p.ldb);
+    auto issue_loads = [&](int step, char *stage) {
+        const int ph = (step >= steps_per_phase) ? 1 : 0;  // at most two phases
+        int c0 = (step - ph * steps_per_phase) * BK;
+        if (EPI != EPI_WGRAD && c0 > c_len - BK) c0 = c_len - BK;
+        const char *Ap = reinterpret_cast<const char *>(p.phases > 1 && ph ? p.A[1] : p.A[0]);
+        const char *Bp = reinterpret_cast<const char *>(
+            (EPI != EPI_SWIGLU && p.phases > 1 && ph) ? p.B[1] : p.B[0]);
+        const char *Bup = reinterpret_cast<const char *>(p.B[1]);
+        char *sa = stage + wave * (A_LOADS * 1024);
+        char *sb = stage + A_BYTES + wave * (B_LOADS * 1024);
+#pragma unroll
+        for (int i = 0; i < A_LOADS; i++) {
+            uint32_t off;  // bytes from the operand base; < 2^32 (checked on the host)
+            if (AKIND == CONTIG) {
+                off = static_cast<uint32_t>(a_off[i] + c0) * 2u;
+            } else {
+                int c = c0 + a_crow[i];
+                if (EPI == EPI_WGRAD) c = min(c, c_len - 1);  // stay in the segment; zeroed below
+                off = static_cast<uint32_t>(a_off[i] + (c_begin + c) * lda32) * 2u;
+            }
+            load16_to_lds(Ap + off, sa + i * 1024);
         }
 #pragma unroll
-        for (int i = 0; i < B_CHUNKS; i++) {
-            const int q = tid + i * NT;
+        for (int i = 0; i < B_LOADS; i++) {
+            uint32_t off;
             if (BKIND == CONTIG) {
-                const int row = q >> 3, ch = q & 7;
-                int64_t n;
-                const uint16_t *Bq = Bp;
-                if (EPI == EPI_SWIGLU) {
-                    // LDS rows alternate 32 gate rows / 32 up rows
-                    const int blk = row >> 5;
-                    n = n0 + (blk >> 1) * 32 + (row & 31);
-                    Bq = (blk & 1) ? p.B[1] : p.B[0];
-                } else {
-                    n = n0 + row;
-                }
-                rb[i] = *reinterpret_cast<const u32x4 *>(Bq + expert * p.strideB + n * p.ldb + c0 + ch * 8);
+                off = static_cast<uint32_t>(b_off[i] + c0) * 2u;
             } else {
-                constexpr int CPR = BN / 8;
-                const int crow = q / CPR, ch = q % CPR;
-                const int64_t c = c0 + crow;
-                if (EPI == EPI_WGRAD) {
-                    if (c < c_len)
-                        rb[i] = *reinterpret_cast<const u32x4 *>(Bp + (c_begin + c) * p.ldb + n0 + ch * 8);
-                    else
-                        rb[i] = u32x4{0, 0, 0, 0};
-                } else {
-                    rb[i] = *reinterpret_cast<const u32x4 *>(Bp + expert * p.strideB + c * p.ldb + n0 + ch * 8);
-                }
+                int c = c0 + b_crow[i];
+                if (EPI == EPI_WGRAD) c = min(c, c_len - 1);
+                off = static_cast<uint32_t>(b_off[i] + (c_begin + c) * ldb32) * 2u;
             }
+            load16_to_lds(((EPI == EPI_SWIGLU && b_up[i]) ? Bup : Bp) + off, sb + i * 1024);
         }
     };
-    auto store_tiles = [&](int stage) {
-        char *sa = smem + stage * STAGE;
-        char *sb = sa + A_BYTES;
+    // wgrad: zero the A c-rows past the end of the expert's rows (after the loads have landed,
+    // before the barrier).  B holds finite in-segment data there, so the products vanish.
+    auto zero_tail = [&](int step, char *stage) {
+        if (EPI != EPI_WGRAD) return;
+        const int c0 = step * BK;
+        if (c0 + BK <= c_len) return;
+        char *sa = stage + wave * (A_LOADS * 1024);
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; i++) {
-            const int q = tid + i * NT;
-            if (AKIND == CONTIG) {
-                *reinterpret_cast<u32x4 *>(sa + contig_off(q >> 3, q & 7)) = ra[i];
-            } else {
-                constexpr int CPR = BM / 8;
-                *reinterpret_cast<u32x4 *>(sa + (q / CPR) * StridedTile<BM>::PITCH + (q % CPR) * 16) = ra[i];
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < B_CHUNKS; i++) {
-            const int q = tid + i * NT;
-            if (BKIND == CONTIG) {
-                *reinterpret_cast<u32x4 *>(sb + contig_off(q >> 3, q & 7)) = rb[i];
-            } else {
-                constexpr int CPR = BN / 8;
-                *reinterpret_cast<u32x4 *>(sb + (q / CPR) * StridedTile<BN>::PITCH + (q % CPR) * 16) = rb[i];
-            }
-        }
+        for (int i = 0; i < A_LOADS; i++)
+            if (c0 + a_crow[i] >= c_len)
+                *reinterpret_cast<u32x4 *>(sa + i * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
     };
 
     f32x16 acc[TM][TN];
@@ -276,43 +320,116 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    if (total_steps > 0) {
-        load_tiles(0);
-        store_tiles(0);
-    }
-    __syncthreads();
-
-    for (int step = 0; step < total_steps; step++) {
-        const int stage = step & 1;
-        if (step + 1 < total_steps) load_tiles(step + 1);
-        const char *sa = smem + stage * STAGE;
-        const char *sb = sa + A_BYTES;
+    // ---- fragment addresses (bytes within a stage), loop-invariant ------------------------------
+    // CONTIG : addr(i, kk) = c_base + i*4096 + c_kofs[kk]      (rows i*32 apart share the swizzle)
+    // STRIDED: addr(i, kk) = s_base[i] + kk*16*R*2 (+ 4*R*2 for the second transposing read)
+    const int lrow32 = lane & 31, g2 = lane >> 5;
+    int c_kofs[BK / 16];
 #pragma unroll
-        for (int kk = 0; kk < BK / 16; kk++) {
-            bf16x8 fa[TM], fb[TN];
+    for (int kk = 0; kk < BK / 16; kk++) c_kofs[kk] = ((kk * 2 + g2) ^ swz(lrow32)) << 4;
+    const int a_cbase = (wm * WM + lrow32) * 128;
+    const int b_cbase = A_BYTES + (wn * WN + lrow32) * 128;
+    int a_sbase[TM], b_sbase[TN];
+    {
+        const int i16 = lane & 15;
+        const int r = i16 >> 2, q = i16 & 3, mb = ((lane >> 4) & 1) * 16;
+        const int cr = 8 * g2 + r;
 #pragma unroll
-            for (int i = 0; i < TM; i++) {
-                if (AKIND == CONTIG)
-                    fa[i] = lds_read_frag_contig(sa, wm * WM + i * 32 + (lane & 31), kk * 2 + (lane >> 5));
-                else
-                    fa[i] = lds_read_frag_strided<BM>(sa, kk * 16, wm * WM + i * 32, lane);
-            }
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                if (BKIND == CONTIG)
-                    fb[j] = lds_read_frag_contig(sb, wn * WN + j * 32 + (lane & 31), kk * 2 + (lane >> 5));
-                else
-                    fb[j] = lds_read_frag_strided<BN>(sb, kk * 16, wn * WN + j * 32, lane);
-            }
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    // operands swapped: the lane then holds 4 consecutive output columns per row
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        for (int i = 0; i < TM; i++) {
+            const int m = wm * WM + i * 32 + mb + 4 * q;
+            a_sbase[i] = strided_off<BM>(cr, m >> 3) + (m & 7) * 2;
         }
-        if (step + 1 < total_steps) store_tiles(stage ^ 1);
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int m = wn * WN + j * 32 + mb + 4 * q;
+            b_sbase[j] = A_BYTES + strided_off<BN>(cr, m >> 3) + (m & 7) * 2;
+        }
+    }
+    typedef __attribute__((ext_vector_type(8))) short s16x8;
+    auto read_a = [&](const char *stage, int i, int kk) -> bf16x8 {
+        if (AKIND == CONTIG) {
+            return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(stage + a_cbase + i * 4096 + c_kofs[kk]));
+        } else {
+            const char *ptr = stage + a_sbase[i] + kk * (16 * BM * 2);
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ptr));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ptr + 4 * BM * 2));
+            return __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+    };
+    auto read_b = [&](const char *stage, int j, int kk) -> bf16x8 {
+        if (BKIND == CONTIG) {
+            return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(stage + b_cbase + j * 4096 + c_kofs[kk]));
+        } else {
+            const char *ptr = stage + b_sbase[j] + kk * (16 * BN * 2);
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ptr));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ptr + 4 * BN * 2));
+            return __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+    };
+
+    // ---- main loop ------------------------------------------------------------------------------
+    // Two LDS stages; the loads of step s+2 are issued as soon as every wavefront has taken its
+    // last fragments of step s out of LDS.  Fragments are double buffered in registers: the reads
+    // of 16-slice kk+1 are interleaved with the MFMAs of slice kk, and the first slice of the next
+    // stage is read under the MFMAs of the last slice of this one, so the wavefront never waits on
+    // LDS latency with an empty MFMA pipe.
+    bf16x8 fa[2][TM], fb[2][TN];
+    auto read_group = [&](const char *stage, int kk, int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[buf][i] = read_a(stage, i, kk);
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[buf][j] = read_b(stage, j, kk);
+    };
+    auto mfma_group = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                // operands swapped: the lane then holds 4 consecutive output columns per row
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+    };
+    // scheduling hint: one LDS read, then one MFMA, ... then the remaining MFMAs
+    constexpr int DS_READS = TM * (AKIND == CONTIG ? 1 : 2) + TN * (BKIND == CONTIG ? 1 : 2);
+    auto interleave = [&]() {
+#pragma unroll
+        for (int r = 0; r < DS_READS; r++) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+        }
+        if (TM * TN > DS_READS) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - DS_READS, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // one contraction step on `cur`; `nxt` holds step s+1 when this returns
+    auto half_step = [&](char *cur, char *nxt, int s) {
+#pragma unroll
+        for (int kk = 0; kk < BK / 16 - 1; kk++) {
+            read_group(cur, kk + 1, (kk + 1) & 1);
+            mfma_group(kk & 1);
+            interleave();
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's loads of step s+1 landed
+        zero_tail(s + 1, nxt);
+        __syncthreads();                     // everyone's did, and nobody reads `cur` any more
+        issue_loads(s + 2, cur);             // past the end on the last steps: harmless re-read
+        read_group(nxt, 0, 0);
+        mfma_group((BK / 16 - 1) & 1);
+        interleave();
+    };
+    // Steps are taken in pairs so the stage names are static; an odd step count (wgrad only: the
+    // host requires kc % 128 == 0 otherwise) is padded with a step whose A tile is all zero.
+    const int loop_steps = (total_steps + 1) & ~1;
+    if (loop_steps > 0) {
+        issue_loads(0, stage0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        zero_tail(0, stage0);
         __syncthreads();
+        issue_loads(1, stage1);
+        read_group(stage0, 0, 0);
+        for (int step = 0; step < loop_steps; step += 2) {
+            half_step(stage0, stage1, step);
+            half_step(stage1, stage0, step + 1);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the trailing loads before LDS is released
     }
 
     // ---- epilogue ------------------------------------------------------------------------------
@@ -401,34 +518,52 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 
 // ---- host side ---------------------------------------------------------------------------------
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI>
-int launch(const GemmParams &p, dim3 grid, hipStream_t st) {
-    constexpr int NT = WAVES_M * WAVES_N * 64;
-    constexpr int lds = 2 * (TileBytes<AKIND, BM>::value + TileBytes<BKIND, BN>::value);
-    auto kern = ggemm_kernel<BM, BN, WAVES_M, WAVES_N, AKIND, BKIND, EPI>;
-    static bool attr_set = false;  // one-time opt-in to > 64 KiB of dynamic LDS
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-            return OM_ERR_LAUNCH;
-        attr_set = true;
-    }
-    kern<<<grid, dim3(NT), lds, st>>>(p);
+// Two tile shapes: 256x256 (wavefront tile 128x128) for the training shapes, 128x128 (wavefront
+// tile 64x64) when an extent is not a multiple of 256 or experts hold few rows each.
+struct Shape { int bm, bn; };
+
+inline bool mult(int64_t v, int m) { return v > 0 && v % m == 0; }
+inline bool fits31(int64_t elems) { return elems >= 0 && elems < (1LL << 31); }
+
+// wavefront grid of the 256x256 tile (overridable for tuning builds)
+#ifndef OM_WAVES_M
+#define OM_WAVES_M 2
+#endif
+#ifndef OM_WAVES_N
+#define OM_WAVES_N 2
+#endif
+template <int BM> struct Waves {
+    static constexpr int M = (BM == 256) ? OM_WAVES_M : 2;
+    static constexpr int N = (BM == 256) ? OM_WAVES_N : 2;
+};
+
+template <int BM, int BN, int AKIND, int BKIND, int EPI>
+int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad family
+    constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
+    p.m_tiles_max = static_cast<int>((rows + BM - 1) / BM + p.n_experts);
+    const int64_t blocks = static_cast<int64_t>(p.m_tiles_max) * (p.n_cols / BN_OUT);
+    if (blocks > 0x7fffffffLL) return OM_ERR_SHAPE;
+    ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI>
+        <<<dim3(static_cast<unsigned>(blocks)), dim3(Waves<BM>::M * Waves<BM>::N * 64), 0, st>>>(p);
     return om_launch_status();
 }
 
-inline bool mult(int64_t v, int m) { return v > 0 && v % m == 0; }
+template <int AKIND, int BKIND, int EPI>
+int launch_rows_auto(GemmParams &p, int64_t rows, hipStream_t st) {
+    constexpr int div = (EPI == EPI_SWIGLU) ? 2 : 1;
+    const bool big_ok = p.n_cols % (256 / div) == 0;
+    const bool few_rows = rows < static_cast<int64_t>(p.n_experts) * 192;
+    if (big_ok && !few_rows) return launch_rows<256, 256, AKIND, BKIND, EPI>(p, rows, st);
+    if (p.n_cols % (128 / div) != 0) return OM_ERR_SHAPE;
+    return launch_rows<128, 128, AKIND, BKIND, EPI>(p, rows, st);
+}
 
 }  // namespace
-
-// Tile shape used by the fwd / dgrad launches.
-#define OM_BM 128
-#define OM_BN 128
 
 extern "C" int om_grouped_gemm_fwd(const void *input, const void *weight, void *output,
                                    const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                    int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(N, OM_BN) || !mult(K, BK)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!input || !weight || !output || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(input) || !om_aligned16(weight) || !om_aligned16(output)) return OM_ERR_ALIGN;
@@ -439,16 +574,15 @@ extern "C" int om_grouped_gemm_fwd(const void *input, const void *weight, void *
     p.cum = cum_token_counts;
     p.lda = K; p.ldb = K; p.ldc = N;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(N) * K;
+    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = N; p.kc = K; p.phases = 1;
-    p.m_tiles_max = static_cast<int>((rows + OM_BM - 1) / OM_BM + G);
-    dim3 grid(static_cast<unsigned>(p.m_tiles_max) * (N / OM_BN));
-    return launch<OM_BM, OM_BN, 2, 2, CONTIG, CONTIG, EPI_STORE>(p, grid, om_stream(stream));
+    return launch_rows_auto<CONTIG, CONTIG, EPI_STORE>(p, rows, om_stream(stream));
 }
 
 extern "C" int om_grouped_gemm_dgrad(const void *output_grad, const void *weight, void *input_grad,
                                      const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                      int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(N, BK) || !mult(K, OM_BN)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!output_grad || !weight || !input_grad || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(output_grad) || !om_aligned16(weight) || !om_aligned16(input_grad)) return OM_ERR_ALIGN;
@@ -459,16 +593,15 @@ extern "C" int om_grouped_gemm_dgrad(const void *output_grad, const void *weight
     p.cum = cum_token_counts;
     p.lda = N; p.ldb = K; p.ldc = K;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(N) * K;
+    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
-    p.m_tiles_max = static_cast<int>((rows + OM_BM - 1) / OM_BM + G);
-    dim3 grid(static_cast<unsigned>(p.m_tiles_max) * (K / OM_BN));
-    return launch<OM_BM, OM_BN, 2, 2, CONTIG, STRIDED, EPI_STORE>(p, grid, om_stream(stream));
+    return launch_rows_auto<CONTIG, STRIDED, EPI_STORE>(p, rows, om_stream(stream));
 }
 
 extern "C" int om_grouped_gemm_wgrad(const void *output_grad, const void *input, void *weight_grad,
                                      const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                      int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(N, OM_BM) || !mult(K, OM_BN)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
     if (!output_grad || !input || !weight_grad || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(output_grad) || !om_aligned16(input) || !om_aligned16(weight_grad)) return OM_ERR_ALIGN;
     GemmParams p = {};
@@ -478,15 +611,25 @@ extern "C" int om_grouped_gemm_wgrad(const void *output_grad, const void *input,
     p.cum = cum_token_counts;
     p.lda = N; p.ldb = K; p.ldc = K;
     p.strideC = w_stride ? w_stride : static_cast<int64_t>(N) * K;
+    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideC * G)) return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
-    dim3 grid(static_cast<unsigned>((N / OM_BM) * (K / OM_BN)), static_cast<unsigned>(G));
-    return launch<OM_BM, OM_BN, 2, 2, STRIDED, STRIDED, EPI_WGRAD>(p, grid, om_stream(stream));
+    hipStream_t st = om_stream(stream);
+    if (N % 256 == 0 && K % 256 == 0) {
+        dim3 grid(static_cast<unsigned>((N / 256) * (K / 256)), static_cast<unsigned>(G));
+        ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD>
+            <<<grid, dim3(Waves<256>::M * Waves<256>::N * 64), 0, st>>>(p);
+    } else {
+        dim3 grid(static_cast<unsigned>((N / 128) * (K / 128)), static_cast<unsigned>(G));
+        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD><<<grid, dim3(256), 0, st>>>(p);
+    }
+    return om_launch_status();
 }
 
 extern "C" int om_merged_mlp_gate_up_fwd(const void *x, const void *w_gate, const void *w_up, void *g,
                                          void *u, void *h, const int32_t *cum_token_counts,
-                                         int64_t rows, int G, int I, int H, int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(I, OM_BN / 2) || !mult(H, BK)) return OM_ERR_SHAPE;
+                                         int64_t rows, int G, int I, int H, int64_t w_stride,
+                                         void *stream) {
+    if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 128)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!x || !w_gate || !w_up || !g || !u || !h || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(x) || !om_aligned16(w_gate) || !om_aligned16(w_up) || !om_aligned16(g) ||
@@ -502,16 +645,16 @@ extern "C" int om_merged_mlp_gate_up_fwd(const void *x, const void *w_gate, cons
     p.cum = cum_token_counts;
     p.lda = H; p.ldb = H; p.ldc = I;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(I) * H;
+    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = I; p.kc = H; p.phases = 1;
-    p.m_tiles_max = static_cast<int>((rows + OM_BM - 1) / OM_BM + G);
-    dim3 grid(static_cast<unsigned>(p.m_tiles_max) * (I / (OM_BN / 2)));
-    return launch<OM_BM, OM_BN, 2, 2, CONTIG, CONTIG, EPI_SWIGLU>(p, grid, om_stream(stream));
+    return launch_rows_auto<CONTIG, CONTIG, EPI_SWIGLU>(p, rows, om_stream(stream));
 }
 
 extern "C" int om_merged_mlp_down_dgrad(const void *dy, const void *w_down, const void *g, const void *u,
                                         void *dg, void *du, const int32_t *cum_token_counts,
-                                        int64_t rows, int G, int I, int H, int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(I, OM_BN) || !mult(H, BK)) return OM_ERR_SHAPE;
+                                        int64_t rows, int G, int I, int H, int64_t w_stride,
+                                        void *stream) {
+    if (rows < 0 || G < 1 || !mult(I, 128) || !mult(H, 128)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!dy || !w_down || !g || !u || !dg || !du || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(dy) || !om_aligned16(w_down) || !om_aligned16(g) || !om_aligned16(u) ||
@@ -527,16 +670,16 @@ extern "C" int om_merged_mlp_down_dgrad(const void *dy, const void *w_down, cons
     p.cum = cum_token_counts;
     p.lda = H; p.ldb = I; p.ldc = I;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(H) * I;
+    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = I; p.kc = H; p.phases = 1;
-    p.m_tiles_max = static_cast<int>((rows + OM_BM - 1) / OM_BM + G);
-    dim3 grid(static_cast<unsigned>(p.m_tiles_max) * (I / OM_BN));
-    return launch<OM_BM, OM_BN, 2, 2, CONTIG, STRIDED, EPI_SWIGLU_BWD>(p, grid, om_stream(stream));
+    return launch_rows_auto<CONTIG, STRIDED, EPI_SWIGLU_BWD>(p, rows, om_stream(stream));
 }
 
 extern "C" int om_merged_mlp_gate_up_dgrad(const void *dg, const void *du, const void *w_gate,
                                            const void *w_up, void *dx, const int32_t *cum_token_counts,
-                                           int64_t rows, int G, int I, int H, int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(I, BK) || !mult(H, OM_BN)) return OM_ERR_SHAPE;
+                                           int64_t rows, int G, int I, int H, int64_t w_stride,
+                                           void *stream) {
+    if (rows < 0 || G < 1 || !mult(I, 128) || !mult(H, 128)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!dg || !du || !w_gate || !w_up || !dx || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(dg) || !om_aligned16(du) || !om_aligned16(w_gate) || !om_aligned16(w_up) ||
@@ -551,8 +694,7 @@ extern "C" int om_merged_mlp_gate_up_dgrad(const void *dg, const void *du, const
     p.cum = cum_token_counts;
     p.lda = I; p.ldb = H; p.ldc = H;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(I) * H;
+    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = H; p.kc = I; p.phases = 2;
-    p.m_tiles_max = static_cast<int>((rows + OM_BM - 1) / OM_BM + G);
-    dim3 grid(static_cast<unsigned>(p.m_tiles_max) * (H / OM_BN));
-    return launch<OM_BM, OM_BN, 2, 2, CONTIG, STRIDED, EPI_STORE>(p, grid, om_stream(stream));
+    return launch_rows_auto<CONTIG, STRIDED, EPI_STORE>(p, rows, om_stream(stream));
 }
