@@ -80,3 +80,136 @@ def test_fast_block_fwd_bwd(cuda, name, scale):
         a = got[k].float().cpu()
         assert mean_rel(a, gref) <= 1e-2, (k, mean_rel(a, gref))
         assert max_abs(a, gref) <= MAX_ABS * max(1.0, float(gref.abs().max())), (k, max_abs(a, gref))
+
+
+def test_fast_block_injected_logits_skewed(cuda):
+    """C4: Zipf-skewed routing injected at the functional level (router logits given): many experts
+    get 0-8 rows, a few get hundreds.  Expert computation only (router excluded), fwd+bwd."""
+    from optimus.models.common.moe import SoftmaxTopkRouterFunction, MergedMLPFunction, expert_computation
+    inp = sc.moe_inputs("C4")
+    c = inp["cfg"]
+    logits = inp["logits"]
+    assert R.min_topk_gap_ulps(torch.softmax(logits, 1), c["K"]) > 4.0
+    w_ref, e_ref, _ = R.olmoe_router(logits, c["K"], False, torch.bfloat16)
+    counts = torch.bincount(e_ref.flatten(), minlength=c["N"])
+    assert int((counts <= 8).sum()) >= 8 and int(counts.max()) >= 200      # the skew the config asks for
+    w, e = SoftmaxTopkRouterFunction.apply(logits.to(cuda), c["K"], False, torch.bfloat16)
+    assert torch.equal(e.cpu(), e_ref)
+    t = {k: inp[k].to(cuda).requires_grad_(True) for k in ("x", "w_gate", "w_up", "w_down")}
+    wd = w.detach().requires_grad_(True)
+    fn = lambda gi, cum: MergedMLPFunction.apply(gi, t["w_gate"], t["w_up"], t["w_down"], cum)
+    out = expert_computation(t["x"], wd, e, 0, c["N"], fn, c["N"])
+    out.backward(inp["dout"].to(cuda))
+    r = {k: inp[k].float().requires_grad_(True) for k in ("x", "w_gate", "w_up", "w_down")}
+    wr = w_ref.float().requires_grad_(True)
+    ref = torch.zeros(c["T"], c["H"])
+    for n in range(c["N"]):
+        tok, kk = torch.where(e_ref == n)
+        if tok.numel():
+            ref = ref.index_add(0, tok, L.expert_mlp(r["x"][tok], r["w_gate"][n], r["w_up"][n], r["w_down"][n]) * wr[tok, kk, None])
+    ref.backward(inp["dout"].float())
+    assert max_abs(out.float().cpu(), ref.detach()) <= MAX_ABS and mean_rel(out.float().cpu(), ref.detach()) <= 4e-3
+    for k in r:
+        assert mean_rel(t[k].grad.float().cpu(), r[k].grad) <= 1e-2, k
+    assert mean_rel(wd.grad.float().cpu(), wr.grad) <= 1e-2
+    empty = counts == 0
+    if empty.any():
+        assert float(t["w_gate"].grad[empty.to(cuda)].abs().max()) == 0.0
+
+
+def test_unmerged_block_matches_merged(cuda):
+    """OlmoeParallelSparseMoeBlock (ModuleList of per-expert Linear weights, the reference's slow
+    block interface) runs the same kernels over a strided view: identical bits to the merged block,
+    and the per-expert parameters receive the gradients."""
+    inp = sc.moe_inputs("C1", scale_tokens=0.5)
+    c = inp["cfg"]
+    # model-dtype router logits in all three (the slow-block twin has no fp32-logits option)
+    a = _olmoe_block(inp, cuda, fast=True, merged=True, fp32_logits=False)
+    b = _olmoe_block(inp, cuda, fast=False, fp32_logits=False)
+    d = _olmoe_block(inp, cuda, fast=True, merged=False, fp32_logits=False)
+    x = inp["x"].to(cuda).view(2, c["T"] // 2, c["H"])
+    outs = []
+    for blk in (a, b, d):
+        xi = x.clone().requires_grad_(True)
+        o, lg = blk(xi)
+        o.backward(inp["dout"].to(cuda).view_as(o))
+        outs.append((o, xi.grad))
+    for o, gx in outs[1:]:
+        assert torch.equal(o, outs[0][0]) and torch.equal(gx, outs[0][1])
+    assert torch.equal(b.experts[3].up_proj.weight.grad, a.experts.up_proj_merged_weight.grad[3])
+    assert torch.equal(d.experts[5].down_proj.weight.grad, a.experts.down_proj_merged_weight.grad[5])
+    # with MixedPrecisionAdamW the per-expert weights alias flat_param and still run without copies
+    from optimus.optimizers import MixedPrecisionAdamW
+    opt = MixedPrecisionAdamW(b.parameters(), b, lr=1e-3, dtype=torch.bfloat16, device=cuda, warmup_steps=10**9)
+    xi = x.clone().requires_grad_(True)
+    o, _ = b(xi)
+    assert torch.equal(o, outs[0][0])
+    o.backward(inp["dout"].to(cuda).view_as(o))
+    assert b.experts[0].gate_proj.weight.grad.data_ptr() == opt.flat_grad.data_ptr() + 2 * opt.param_start_inds[1]
+    opt.step()
+
+
+def test_activation_checkpointing_recomputes_identically(cuda):
+    inp = sc.moe_inputs("C1", scale_tokens=0.25)
+    c = inp["cfg"]
+    a = _olmoe_block(inp, cuda)
+    b = _olmoe_block(inp, cuda)
+    b.use_activation_checkpointing_for_moe = 1
+    res = []
+    for blk in (a, b):
+        xi = inp["x"].to(cuda).view(1, c["T"], c["H"]).requires_grad_(True)
+        o, _ = blk(xi)
+        o.backward(inp["dout"].to(cuda).view_as(o))
+        res.append((o, xi.grad, blk.experts.gate_proj_merged_weight.grad))
+    for x0, x1 in zip(*res):
+        assert torch.equal(x0, x1)
+
+
+@pytest.mark.parametrize("ep_ind", [0, 3])
+def test_dsv3_block_one_rank_share(cuda, ep_ind):
+    """C5 at reduced size: DeepseekV3ParallelMoE with expert_parallelism=8 (32 of 256 routed experts
+    local) + shared expert, against the fp32 restatement of the reference block."""
+    from optimus.mapper import ParallelDpPpEpTpMapper
+    from optimus.models.deepseek_v3.configuration_deepseek_v3 import DeepseekV3ParallelConfig
+    from optimus.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3ParallelMoE
+    inp = sc.dsv3_inputs(scale_tokens=1 / 16, scale_hidden=1 / 7)
+    c = inp["cfg"]
+    cfg = DeepseekV3ParallelConfig(hidden_size=c["H"], moe_intermediate_size=c["I"], n_routed_experts=c["N"],
+                                   n_group=c["n_group"], topk_group=c["topk_group"], num_experts_per_tok=c["K"],
+                                   expert_parallelism=8)
+    pmap = ParallelDpPpEpTpMapper(expert_parallelism=8, rank=ep_ind)
+    assert pmap.ep_ind == ep_ind
+    blk = DeepseekV3ParallelMoE(cfg, pmap).to(cuda).to(torch.bfloat16)
+    with torch.no_grad():
+        blk.gate.weight.copy_(inp["router_w"])
+        blk.gate.e_score_correction_bias.copy_(inp["bias"])
+        for e, m in enumerate(blk.experts):
+            m.gate_proj.weight.copy_(inp["w_gate"][e]); m.up_proj.weight.copy_(inp["w_up"][e])
+            m.down_proj.weight.copy_(inp["w_down"][e])
+        blk.shared_experts.gate_proj.weight.copy_(inp["ws_gate"]); blk.shared_experts.up_proj.weight.copy_(inp["ws_up"])
+        blk.shared_experts.down_proj.weight.copy_(inp["ws_down"])
+    x = inp["x"].to(cuda).view(2, c["T"] // 2, c["H"]).requires_grad_(True)
+    out = blk(x)
+    out.backward(inp["dout"].to(cuda).view_as(out))
+    # reference in fp32 on the same (bf16-rounded) values; router weight as the module holds it
+    rw = blk.gate.weight.detach().float().cpu()
+    names = ("x", "w_gate", "w_up", "w_down", "ws_gate", "ws_up", "ws_down")
+    t = {k: inp[k].float().requires_grad_(True) for k in names}
+    rwt = rw.clone().requires_grad_(True)
+    bias = blk.gate.e_score_correction_bias.detach().float().cpu()
+    ref, e_ref, w_ref = L.dsv3_moe_block(t["x"], rwt, bias, t["w_gate"], t["w_up"], t["w_down"], t["ws_gate"],
+                                         t["ws_up"], t["ws_down"], c["n_group"], c["topk_group"], c["K"], True, 2.5,
+                                         expert_start_idx=ep_ind * c["NR"])
+    ref.backward(inp["dout"].float())
+    # routing: same expert sets per token (the reference leaves the order unspecified)
+    e_gpu, _ = blk.gate(x.detach())
+    same = (torch.sort(e_gpu.cpu(), 1).values == torch.sort(e_ref, 1).values).all(1)
+    assert float(same.float().mean()) >= 0.999       # fp32 GEMM summation order can flip a near-tie
+    o = out.float().cpu().view(c["T"], c["H"])[same]
+    assert max_abs(o, ref.detach()[same]) <= MAX_ABS and mean_rel(o, ref.detach()[same]) <= 4e-3
+    if bool(same.all()):
+        assert mean_rel(x.grad.float().cpu().view(c["T"], c["H"]), t["x"].grad) <= 1e-2
+        assert mean_rel(blk.shared_experts.up_proj.weight.grad.float().cpu(), t["ws_up"].grad) <= 1e-2
+        got = torch.stack([m.down_proj.weight.grad for m in blk.experts]).float().cpu()
+        assert mean_rel(got, t["w_down"].grad) <= 1e-2
+        assert mean_rel(blk.gate.weight.grad.float().cpu(), rwt.grad) <= 2e-2

@@ -1,0 +1,86 @@
+"""Pins the router restatements (oracle/routing.py) against the library calls the reference makes
+(torch.softmax, torch.topk) on tie-free rows, their invariants, and a brute-force statement of the
+DeepSeek-V3 group-limited selection on a tiny shape."""
+import itertools
+
+import pytest
+import torch
+
+from oracle import routing as R
+
+
+@pytest.mark.parametrize("T,N,K,renorm", [(512, 8, 2, True), (2048, 64, 8, False), (256, 256, 8, True)])
+def test_olmoe_router_equals_torch_topk_on_tie_free_rows(T, N, K, renorm):
+    logits = torch.randn(T, N, generator=torch.Generator().manual_seed(N))
+    assert R.min_topk_gap_ulps(torch.softmax(logits, 1), K) > 4.0
+    w, e, p = R.olmoe_router(logits, K, renorm, torch.float32)
+    tw, te = torch.topk(torch.softmax(logits, dim=1, dtype=torch.float), K, dim=-1)   # moe.py:467-468
+    if renorm:
+        tw = tw / tw.sum(dim=-1, keepdim=True)
+    assert torch.equal(e, te) and torch.equal(w, tw)
+    assert bool((w[:, :-1] >= w[:, 1:]).all())
+    assert bool((torch.sort(e, 1).values[:, 1:] != torch.sort(e, 1).values[:, :-1]).all())
+    if renorm:
+        assert torch.allclose(w.sum(1), torch.ones(T), atol=1e-6)
+
+
+def test_tie_break_is_lowest_index_first():
+    logits = torch.zeros(4, 16)
+    logits[1, 5:9] = 1.0
+    _, e, _ = R.olmoe_router(logits, 3, False, torch.float32)
+    assert e[0].tolist() == [0, 1, 2] and e[1].tolist() == [5, 6, 7]
+
+
+def test_gap_metric_flags_near_ties():
+    p = torch.tensor([[0.5, 0.25, 0.25 * (1 + 2 ** -23), 0.0]])
+    assert R.min_topk_gap_ulps(p, 2) <= 1.0
+    assert R.min_topk_gap_ulps(torch.tensor([[0.5, 0.3, 0.2]]), 2) > 1e5
+
+
+def _dsv3_brute(scores, bias, n_group, topk_group, K):
+    """Direct statement of modeling_deepseek_v3.py:164-180 with python loops."""
+    T, N = scores.shape
+    gs = N // n_group
+    out = []
+    for t in range(T):
+        c = [float(scores[t, i] + bias[i]) for i in range(N)]
+        gsc = []
+        for g in range(n_group):
+            top2 = sorted(c[g * gs:(g + 1) * gs], reverse=True)[:2]
+            gsc.append(sum(top2))
+        keep = sorted(range(n_group), key=lambda g: (-gsc[g], g))[:topk_group]
+        masked = [c[i] if (i // gs) in keep else 0.0 for i in range(N)]
+        out.append(sorted(range(N), key=lambda i: (-masked[i], i))[:K])
+    return torch.tensor(out)
+
+
+def test_dsv3_group_limited_topk_brute_force():
+    g = torch.Generator().manual_seed(0)
+    scores = torch.rand(200, 16, generator=g)
+    bias = torch.randn(16, generator=g) * 0.1
+    e, _ = R.dsv3_topk_indices(scores, bias, 4, 2, 2)
+    # fp32 sums in the restatement vs python floats here: compare as sets where group scores are
+    # not within rounding of each other (always true for this seed)
+    assert torch.equal(torch.sort(e, 1).values, torch.sort(_dsv3_brute(scores, bias, 4, 2, 2), 1).values)
+
+
+def test_dsv3_router_invariants_and_library_topk():
+    g = torch.Generator().manual_seed(1)
+    T, H, N = 300, 64, 256
+    x = torch.randn(T, H, generator=g); W = torch.randn(N, H, generator=g) * 0.06
+    bias = torch.randn(N, generator=g) * 0.1
+    e, w, logits = R.dsv3_router(x, W, bias, 8, 4, 8, True, 2.5)
+    assert torch.allclose(w.sum(1), torch.full((T,), 2.5), atol=1e-5)
+    scores = logits.sigmoid()
+    # selected experts lie in at most topk_group groups and weights are the un-biased scores
+    assert int((e // 32).sort(1).values.diff(dim=1).ne(0).sum(1).max()) + 1 <= 4
+    ww = scores.gather(1, e); ww = ww / (ww.sum(-1, keepdim=True) + 1e-20) * 2.5
+    assert torch.allclose(w, ww)
+    # same sets as the reference's sequence of torch.topk calls (sorted=False there)
+    sfc = scores + bias
+    group_scores = sfc.view(T, 8, 32).topk(2, dim=-1)[0].sum(dim=-1)
+    group_idx = torch.topk(group_scores, k=4, dim=-1, sorted=False)[1]
+    mask = torch.zeros_like(group_scores).scatter_(1, group_idx, 1)
+    score_mask = mask.unsqueeze(-1).expand(-1, 8, 32).reshape(T, N)
+    ref = torch.topk(sfc.masked_fill(~score_mask.bool(), 0.0), k=8, dim=-1, sorted=False)[1]
+    assert torch.equal(torch.sort(e, 1).values, torch.sort(ref, 1).values)
