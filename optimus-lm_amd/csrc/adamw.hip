@@ -26,69 +26,63 @@ __device__ __forceinline__ void adam_update(float g, float &m, float &v, float &
     m = mm; v = vv; w = ww;
 }
 
-template <typename V> __device__ __forceinline__ V ld_stream(const V *p) {
-    return __builtin_nontemporal_load(p);
-}
-template <typename V> __device__ __forceinline__ void st_stream(V *p, V v) {
-    __builtin_nontemporal_store(v, p);
-}
-
-// bf16 mode: a thread owns 8 consecutive elements per chunk (16 B of grad/param, 2x16 B of
-// each fp32 state); a block owns UNROLL consecutive chunks-of-256-threads so UNROLL x 7 loads
-// are in flight per thread before the first use.
+// bf16 mode: a thread owns 4 consecutive elements per chunk (8 B of grad/param, one 16 B vector of
+// each fp32 state), so every wavefront access is one contiguous span; a block owns UNROLL
+// consecutive chunks so UNROLL x 4 loads are in flight per thread before the first use.  Plain
+// (cached) loads and stores measured faster than nontemporal ones on MI355X for this mix of five
+// read and four write streams.
+#ifndef OM_ADAMW_UNROLL
+#define OM_ADAMW_UNROLL 4
+#endif
 template <int UNROLL>
 __global__ __launch_bounds__(256) void adamw_bf16_kernel(uint16_t *__restrict__ param,
-                                                         const uint16_t *__restrict__ grad,
-                                                         float *__restrict__ master,
-                                                         float *__restrict__ exp_avg,
-                                                         float *__restrict__ exp_avg_sq,
-                                                         int64_t n_vec8, AdamScalars s) {
+                                                            const uint16_t *__restrict__ grad,
+                                                            float *__restrict__ master,
+                                                            float *__restrict__ exp_avg,
+                                                            float *__restrict__ exp_avg_sq,
+                                                            int64_t n_vec4, AdamScalars s) {
     const int64_t base = (static_cast<int64_t>(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
-    u32x4 gq[UNROLL];
-    f32x4 m0[UNROLL], m1[UNROLL], v0[UNROLL], v1[UNROLL], w0[UNROLL], w1[UNROLL];
+    u32x2 gq[UNROLL];
+    f32x4 m0[UNROLL], v0[UNROLL], w0[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
         const int64_t c = base + static_cast<int64_t>(u) * 256;
-        if (c < n_vec8) {
-            gq[u] = ld_stream(reinterpret_cast<const u32x4 *>(grad) + c);
-            m0[u] = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg) + 2 * c);
-            m1[u] = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg) + 2 * c + 1);
-            v0[u] = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg_sq) + 2 * c);
-            v1[u] = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg_sq) + 2 * c + 1);
-            w0[u] = ld_stream(reinterpret_cast<const f32x4 *>(master) + 2 * c);
-            w1[u] = ld_stream(reinterpret_cast<const f32x4 *>(master) + 2 * c + 1);
+        if (c < n_vec4) {
+            gq[u] = *(reinterpret_cast<const u32x2 *>(grad) + c);
+            m0[u] = *(reinterpret_cast<const f32x4 *>(exp_avg) + c);
+            v0[u] = *(reinterpret_cast<const f32x4 *>(exp_avg_sq) + c);
+            w0[u] = *(reinterpret_cast<const f32x4 *>(master) + c);
         }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
         const int64_t c = base + static_cast<int64_t>(u) * 256;
-        if (c < n_vec8) {
-            float g[8];
-            Elem<uint16_t>::unpack(gq[u], g);
-            float w[8];
+        if (c < n_vec4) {
+            float g[4];
+            g[0] = __uint_as_float(gq[u][0] << 16);
+            g[1] = __uint_as_float(gq[u][0] & 0xffff0000u);
+            g[2] = __uint_as_float(gq[u][1] << 16);
+            g[3] = __uint_as_float(gq[u][1] & 0xffff0000u);
+            float w[4];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float ma = m0[u][i], va = v0[u][i], wa = w0[u][i];
-                float mb = m1[u][i], vb = v1[u][i], wb = w1[u][i];
                 adam_update(g[i], ma, va, wa, s);
-                adam_update(g[4 + i], mb, vb, wb, s);
                 m0[u][i] = ma; v0[u][i] = va; w0[u][i] = wa;
-                m1[u][i] = mb; v1[u][i] = vb; w1[u][i] = wb;
                 w[i] = wa;
-                w[4 + i] = wb;
             }
-            st_stream(reinterpret_cast<f32x4 *>(exp_avg) + 2 * c, m0[u]);
-            st_stream(reinterpret_cast<f32x4 *>(exp_avg) + 2 * c + 1, m1[u]);
-            st_stream(reinterpret_cast<f32x4 *>(exp_avg_sq) + 2 * c, v0[u]);
-            st_stream(reinterpret_cast<f32x4 *>(exp_avg_sq) + 2 * c + 1, v1[u]);
-            st_stream(reinterpret_cast<f32x4 *>(master) + 2 * c, w0[u]);
-            st_stream(reinterpret_cast<f32x4 *>(master) + 2 * c + 1, w1[u]);
-            st_stream(reinterpret_cast<u32x4 *>(param) + c, Elem<uint16_t>::pack(w));
+            *(reinterpret_cast<f32x4 *>(exp_avg) + c) = m0[u];
+            *(reinterpret_cast<f32x4 *>(exp_avg_sq) + c) = v0[u];
+            *(reinterpret_cast<f32x4 *>(master) + c) = w0[u];
+            u32x2 pk;
+            pk[0] = static_cast<uint32_t>(f32_to_bf16_bits(w[0])) | (static_cast<uint32_t>(f32_to_bf16_bits(w[1])) << 16);
+            pk[1] = static_cast<uint32_t>(f32_to_bf16_bits(w[2])) | (static_cast<uint32_t>(f32_to_bf16_bits(w[3])) << 16);
+            *(reinterpret_cast<u32x2 *>(param) + c) = pk;
         }
     }
 }
 
-// Elements past the last full vector of 8 (at most 7), and the whole buffer in fp32 mode's tail.
+// Elements past the last full vector of 4 (at most 3).
 __global__ void adamw_bf16_tail_kernel(uint16_t *param, const uint16_t *grad, float *master,
                                        float *exp_avg, float *exp_avg_sq, int64_t start, int64_t n,
                                        AdamScalars s) {
@@ -113,19 +107,19 @@ __global__ __launch_bounds__(256) void adamw_f32_kernel(float *__restrict__ mast
     for (int u = 0; u < UNROLL; u++) {
         const int64_t c = base + static_cast<int64_t>(u) * 256;
         if (c < n_vec4) {
-            f32x4 g = ld_stream(reinterpret_cast<const f32x4 *>(grad) + c);
-            f32x4 m = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg) + c);
-            f32x4 v = ld_stream(reinterpret_cast<const f32x4 *>(exp_avg_sq) + c);
-            f32x4 w = ld_stream(reinterpret_cast<const f32x4 *>(master) + c);
+            f32x4 g = *(reinterpret_cast<const f32x4 *>(grad) + c);
+            f32x4 m = *(reinterpret_cast<const f32x4 *>(exp_avg) + c);
+            f32x4 v = *(reinterpret_cast<const f32x4 *>(exp_avg_sq) + c);
+            f32x4 w = *(reinterpret_cast<const f32x4 *>(master) + c);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float ma = m[i], va = v[i], wa = w[i];
                 adam_update(g[i], ma, va, wa, s);
                 m[i] = ma; v[i] = va; w[i] = wa;
             }
-            st_stream(reinterpret_cast<f32x4 *>(exp_avg) + c, m);
-            st_stream(reinterpret_cast<f32x4 *>(exp_avg_sq) + c, v);
-            st_stream(reinterpret_cast<f32x4 *>(master) + c, w);
+            *(reinterpret_cast<f32x4 *>(exp_avg) + c) = m;
+            *(reinterpret_cast<f32x4 *>(exp_avg_sq) + c) = v;
+            *(reinterpret_cast<f32x4 *>(master) + c) = w;
         }
     }
 }
@@ -169,9 +163,9 @@ extern "C" int om_adamw_step(void *param, const void *grad, float *master, float
     s.use_wd = weight_decay > 0.0 ? 1 : 0;
 
     hipStream_t st = om_stream(stream);
-    constexpr int UNROLL = 2;
+    constexpr int UNROLL = OM_ADAMW_UNROLL;
     if (param_dtype == OM_BF16) {
-        const int64_t n_vec = n / 8;
+        const int64_t n_vec = n / 4;
         if (n_vec > 0) {
             const int64_t blocks = (n_vec + 256 * UNROLL - 1) / (256 * UNROLL);
             if (blocks > 0x7fffffffLL) return OM_ERR_SHAPE;
@@ -179,10 +173,10 @@ extern "C" int om_adamw_step(void *param, const void *grad, float *master, float
                 static_cast<uint16_t *>(param), static_cast<const uint16_t *>(grad), master, exp_avg,
                 exp_avg_sq, n_vec, s);
         }
-        if (n_vec * 8 < n)
+        if (n_vec * 4 < n)
             adamw_bf16_tail_kernel<<<1, 64, 0, st>>>(static_cast<uint16_t *>(param),
                                                      static_cast<const uint16_t *>(grad), master,
-                                                     exp_avg, exp_avg_sq, n_vec * 8, n, s);
+                                                     exp_avg, exp_avg_sq, n_vec * 4, n, s);
     } else {
         const int64_t n_vec = n / 4;
         if (n_vec > 0) {

@@ -186,10 +186,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     int n0;                          // first output column (LDS B row 0)
     int c_begin, c_len;              // contraction range
     if (EPI == EPI_WGRAD) {
-        // grid: x = (N/BM) * (K/BN) tiles of dW[g], y = expert
+        // grid: x = (N/BM) * (K/BN) tiles of dW[g], y = expert; remapped so that an XCD works on
+        // whole experts (all tiles of dW[g] share the expert's rows of both operands)
         const int tiles_n = p.n_cols / BN;
-        expert = blockIdx.y;
-        const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+        const int tiles_e = gridDim.x;
+        const int logical = xcd_remap(blockIdx.y * tiles_e + blockIdx.x, tiles_e * gridDim.y);
+        expert = logical / tiles_e;
+        const int tile = logical - expert * tiles_e;
+        const int tm = tile / tiles_n, tn = tile % tiles_n;
         row_begin = tm * BM;  // row of dW
         row_end = 0;
         n0 = tn * BN;
