@@ -437,86 +437,126 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     }
 
     // ---- epilogue ------------------------------------------------------------------------------
-    // accumulator element r of lane l: output row (l % 32), column (r/4)*8 + (l/32)*4 + (r%4).
+    // Accumulator element r of lane l is output row (l % 32), column (r/4)*8 + (l/32)*4 + (r%4) of
+    // its 32x32 block: a lane holds 4 consecutive columns of ONE row, and the 64 lanes of a store
+    // would touch 32 different rows.  Each wavefront therefore turns its results around through a
+    // private LDS strip (32 rows x COLS bf16, row pitch COLS*2+8 bytes so that both the 8-byte
+    // writes in accumulator layout and the 8-byte reads in row layout are conflict-free) and moves
+    // 16 bytes per lane to and from global memory, 64 lanes covering whole 256-byte row segments.
+    // The fused SwiGLU backward reads g and u in the same row layout.
+    __syncthreads();  // the stages are dead: reuse them as strips
+    constexpr int COLS = (EPI == EPI_SWIGLU) ? WN / 2 : WN;   // output columns of this wavefront
+    constexpr int PITCH = COLS * 2 + 8;
+    constexpr int STRIP = 32 * PITCH;
+    constexpr int NSTRIP = (EPI == EPI_SWIGLU) ? 3 : 1;
+    static_assert(NW * NSTRIP * STRIP <= A_BYTES + B_BYTES, "strips must fit in one stage");
+    char *strip = stage0 + wave * (NSTRIP * STRIP);
     const int lrow = lane & 31;
     const int lcol = (lane >> 5) * 4;
-    if (EPI == EPI_STORE || EPI == EPI_WGRAD) {
-        uint16_t *Cb = p.C + (EPI == EPI_WGRAD ? expert * p.strideC : 0);
+    constexpr int CPRW = COLS / 8;            // 16-byte chunks per strip row
+    constexpr int ITS = 32 * CPRW / 64;       // chunks per lane per strip
+    // write 4 consecutive columns (as bf16) of row lrow at column `col` of strip `which`
+    auto strip_put = [&](int which, int col, float v0, float v1, float v2, float v3) {
+        u32x2 v;
+        v[0] = pack2_bf16(v0, v1);
+        v[1] = pack2_bf16(v2, v3);
+        *reinterpret_cast<u32x2 *>(strip + which * STRIP + lrow * PITCH + col * 2) = v;
+    };
+    auto strip_get = [&](int which, int row, int cc) -> u32x4 {
+        const char *q = strip + which * STRIP + row * PITCH + cc * 16;
+        const u32x2 lo = *reinterpret_cast<const u32x2 *>(q);
+        const u32x2 hi = *reinterpret_cast<const u32x2 *>(q + 8);
+        return u32x4{lo[0], lo[1], hi[0], hi[1]};
+    };
+    auto strip_sync = [&]() {  // LDS operations of one wavefront are performed in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    const int col0 = (EPI == EPI_SWIGLU) ? n0 + (wn * WN) / 2 : n0 + wn * WN;   // first output column
+    uint16_t *Cb = p.C + (EPI == EPI_WGRAD ? expert * p.strideC : 0);
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
-            const int64_t m = static_cast<int64_t>(row_begin) + wm * WM + i * 32 + lrow;
-            if (EPI == EPI_STORE && m >= row_end) continue;
+    for (int i = 0; i < TM; i++) {
+        const int64_t m0 = static_cast<int64_t>(row_begin) + wm * WM + i * 32;  // first row of the strip
+        if (EPI == EPI_SWIGLU) {
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
+            for (int j = 0; j < TN; j += 2)
 #pragma unroll
                 for (int rq = 0; rq < 4; rq++) {
-                    const int n = n0 + wn * WN + j * 32 + rq * 8 + lcol;
-                    u32x2 v;
-                    v[0] = pack2_bf16(acc[i][j][rq * 4 + 0], acc[i][j][rq * 4 + 1]);
-                    v[1] = pack2_bf16(acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3]);
-                    *reinterpret_cast<u32x2 *>(Cb + m * p.ldc + n) = v;
-                }
-            }
-        }
-    } else if (EPI == EPI_SWIGLU) {
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-            const int64_t m = static_cast<int64_t>(row_begin) + wm * WM + i * 32 + lrow;
-            if (m >= row_end) continue;
-#pragma unroll
-            for (int j = 0; j < TN; j += 2) {
-#pragma unroll
-                for (int rq = 0; rq < 4; rq++) {
-                    const int n = n0 + (wn * WN + j * 32) / 2 + rq * 8 + lcol;
                     float hv[4];
 #pragma unroll
                     for (int x = 0; x < 4; x++) {
                         const float gv = acc[i][j][rq * 4 + x], uv = acc[i][j + 1][rq * 4 + x];
                         hv[x] = (gv / (1.0f + __expf(-gv))) * uv;
                     }
-                    u32x2 vg, vu, vh;
-                    vg[0] = pack2_bf16(acc[i][j][rq * 4 + 0], acc[i][j][rq * 4 + 1]);
-                    vg[1] = pack2_bf16(acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3]);
-                    vu[0] = pack2_bf16(acc[i][j + 1][rq * 4 + 0], acc[i][j + 1][rq * 4 + 1]);
-                    vu[1] = pack2_bf16(acc[i][j + 1][rq * 4 + 2], acc[i][j + 1][rq * 4 + 3]);
-                    vh[0] = pack2_bf16(hv[0], hv[1]);
-                    vh[1] = pack2_bf16(hv[2], hv[3]);
-                    *reinterpret_cast<u32x2 *>(p.C + m * p.ldc + n) = vg;
-                    *reinterpret_cast<u32x2 *>(p.C1 + m * p.ldc + n) = vu;
-                    *reinterpret_cast<u32x2 *>(p.C2 + m * p.ldc + n) = vh;
+                    const int col = (j / 2) * 32 + rq * 8 + lcol;
+                    strip_put(0, col, acc[i][j][rq * 4], acc[i][j][rq * 4 + 1], acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3]);
+                    strip_put(1, col, acc[i][j + 1][rq * 4], acc[i][j + 1][rq * 4 + 1], acc[i][j + 1][rq * 4 + 2], acc[i][j + 1][rq * 4 + 3]);
+                    strip_put(2, col, hv[0], hv[1], hv[2], hv[3]);
+                }
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++)
+                    strip_put(0, j * 32 + rq * 8 + lcol, acc[i][j][rq * 4], acc[i][j][rq * 4 + 1],
+                              acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3]);
+        }
+        strip_sync();
+        if (EPI == EPI_SWIGLU_BWD) {
+            u32x4 gq[ITS], uq[ITS];
+#pragma unroll
+            for (int it = 0; it < ITS; it++) {
+                const int q = it * 64 + lane;
+                const int64_t m = m0 + q / CPRW;
+                if (m < row_end) {
+                    const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
+                    gq[it] = *reinterpret_cast<const u32x4 *>(p.G + o);
+                    uq[it] = *reinterpret_cast<const u32x4 *>(p.U + o);
                 }
             }
-        }
-    } else {  // EPI_SWIGLU_BWD
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
-            const int64_t m = static_cast<int64_t>(row_begin) + wm * WM + i * 32 + lrow;
-            if (m >= row_end) continue;
+            for (int it = 0; it < ITS; it++) {
+                const int q = it * 64 + lane;
+                const int64_t m = m0 + q / CPRW;
+                if (m < row_end) {
+                    float dh[8], gv[8], uv[8], dg[8], du[8];
+                    Elem<uint16_t>::unpack(strip_get(0, q / CPRW, q % CPRW), dh);
+                    Elem<uint16_t>::unpack(gq[it], gv);
+                    Elem<uint16_t>::unpack(uq[it], uv);
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-#pragma unroll
-                for (int rq = 0; rq < 4; rq++) {
-                    const int n = n0 + wn * WN + j * 32 + rq * 8 + lcol;
-                    float gv[4], uv[4], dg[4], du[4];
-                    unpack4_bf16(*reinterpret_cast<const u32x2 *>(p.G + m * p.ldc + n), gv);
-                    unpack4_bf16(*reinterpret_cast<const u32x2 *>(p.U + m * p.ldc + n), uv);
+                    for (int x = 0; x < 8; x++) {
+                        const float sg = 1.0f / (1.0f + __expf(-gv[x]));
+                        du[x] = dh[x] * (gv[x] * sg);
+                        dg[x] = (dh[x] * uv[x]) * (sg * (1.0f + gv[x] * (1.0f - sg)));
+                    }
+                    const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
+                    u32x4 vg, vu;
 #pragma unroll
                     for (int x = 0; x < 4; x++) {
-                        const float dh = acc[i][j][rq * 4 + x];
-                        const float sg = 1.0f / (1.0f + __expf(-gv[x]));
-                        du[x] = dh * (gv[x] * sg);
-                        dg[x] = (dh * uv[x]) * (sg * (1.0f + gv[x] * (1.0f - sg)));
+                        vg[x] = pack2_bf16(dg[2 * x], dg[2 * x + 1]);
+                        vu[x] = pack2_bf16(du[2 * x], du[2 * x + 1]);
                     }
-                    u32x2 vg, vu;
-                    vg[0] = pack2_bf16(dg[0], dg[1]);
-                    vg[1] = pack2_bf16(dg[2], dg[3]);
-                    vu[0] = pack2_bf16(du[0], du[1]);
-                    vu[1] = pack2_bf16(du[2], du[3]);
-                    *reinterpret_cast<u32x2 *>(p.C + m * p.ldc + n) = vg;
-                    *reinterpret_cast<u32x2 *>(p.C1 + m * p.ldc + n) = vu;
+                    *reinterpret_cast<u32x4 *>(p.C + o) = vg;
+                    *reinterpret_cast<u32x4 *>(p.C1 + o) = vu;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < ITS; it++) {
+                const int q = it * 64 + lane;
+                const int64_t m = m0 + q / CPRW;
+                if (EPI == EPI_WGRAD || m < row_end) {
+                    const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
+                    *reinterpret_cast<u32x4 *>(Cb + o) = strip_get(0, q / CPRW, q % CPRW);
+                    if (EPI == EPI_SWIGLU) {
+                        *reinterpret_cast<u32x4 *>(p.C1 + o) = strip_get(1, q / CPRW, q % CPRW);
+                        *reinterpret_cast<u32x4 *>(p.C2 + o) = strip_get(2, q / CPRW, q % CPRW);
+                    }
                 }
             }
         }
+        strip_sync();  // the strip is rewritten by the next i
     }
 }
 
