@@ -574,7 +574,7 @@ inline bool fits31(int64_t elems) { return elems >= 0 && elems < (1LL << 31); }
 #define OM_WAVES_M 2
 #endif
 #ifndef OM_WAVES_N
-#define OM_WAVES_N 2
+#define OM_WAVES_N 4
 #endif
 template <int BM> struct Waves {
     static constexpr int M = (BM == 256) ? OM_WAVES_M : 2;
