@@ -27,6 +27,17 @@ sys.path.insert(0, os.path.join(ROOT, "optimus-lm_amd"))
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM bytes per launch (read + write) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same
+# command, scaled by what the counters read for a plain 1 GiB copy (x2.000 and x1.000); the table
+# and the commands are in profiles/hbm_traffic_c3_expert_gemms_and_c2_adamw.md.  Offline figures:
+# counters cannot be collected inside the timed run.
+MIB = float(1 << 20)
+MEASURED_TRAFFIC_BYTES = {
+    "om_merged_mlp_gate_up_fwd": (2388 + 769) * MIB, "om_grouped_gemm_fwd": (1132 + 512) * MIB,
+    "om_grouped_gemm_wgrad": (830 + 256) * MIB, "om_merged_mlp_down_dgrad": (1718 + 512) * MIB,
+    "om_merged_mlp_gate_up_dgrad": (2101 + 512) * MIB, "om_adamw_step": (92125 + 92125) * MIB,
+}
+
 GEMM_ENTRY_PRODUCTS = {     # C-ABI entry -> number of [rows x N x K] products per launch
     "om_merged_mlp_gate_up_fwd": 2, "om_grouped_gemm_fwd": 1, "om_grouped_gemm_wgrad": 1,
     "om_merged_mlp_down_dgrad": 1, "om_merged_mlp_gate_up_dgrad": 2, "om_grouped_gemm_dgrad": 1,
@@ -96,7 +107,7 @@ def bench_moe(args, device):
     achieved = GEMM_ENTRY_PRODUCTS[dom] * prod_flops / dom_avg_s / 1e12
     roofline = {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1),
                 "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                "traffic": None,
+                "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
                 "all_expert_gemms": {"flops_per_step": 9 * prod_flops, "ms_per_step": round(gemm_ms, 3),
                                      "achieved": round(9 * prod_flops / (gemm_ms * 1e-3) / 1e12, 1),
                                      "frac": round(9 * prod_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}}
@@ -151,13 +162,20 @@ def bench_adamw(args, device):
                     hp["step_id"] + 1 + i, hp["lr"], hp["betas"][0], hp["betas"][1], hp["eps"],
                     hp["weight_decay"])
 
-    for i in range(2):
-        step(i)
+    # the memory clocks take a few seconds of load to reach their steady state after the idle
+    # period of the CPU baseline: warm up untimed for about three seconds
+    t_warm = time.perf_counter()
+    i = 0
+    while i < args.warmup or time.perf_counter() - t_warm < 3.0:
+        step(i % 30)
+        i += 1
+        if i % 10 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     _native.launch_log = []
     t0 = time.perf_counter()
     for i in range(steps):
-        step(2 + i)
+        step(40 + i)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     log, _native.launch_log = _native.launch_log, None
@@ -172,7 +190,7 @@ def bench_adamw(args, device):
                                    "param/grad + fp32 master/m/v, step 100"},
             "roofline": {"bound": "hbm", "kernel": "om_adamw_step", "achieved": round(gbs, 1),
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
-                         "traffic": None, "bytes_per_param": 28, "kernel_avg_ms": round(avg_s * 1e3, 3)}}
+                         "traffic": MEASURED_TRAFFIC_BYTES["om_adamw_step"], "bytes_per_param": 28, "kernel_avg_ms": round(avg_s * 1e3, 3)}}
 
 
 def cpu_baseline_adamw():
