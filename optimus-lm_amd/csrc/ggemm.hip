@@ -70,7 +70,9 @@ __device__ __forceinline__ void load16_to_lds(const void *gptr, char *lds_base) 
 }
 
 // ---- CONTIG tile: R rows x 64 c; 128-byte rows; chunk position = chunk ^ swz(row) ----------
-__device__ __forceinline__ int swz(int row) { return ((row & 31) + ((row & 31) >> 3)) & 7; }  // period 32
+// (row >> 1) & 7: measured conflict-free for ds_read_b128 with 32 consecutive rows per half-wave
+// (counter SQ_LDS_BANK_CONFLICT = 0, 4 cycles per read); period 16, so rows 32 apart share it.
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 __device__ __forceinline__ int contig_off(int row, int ch) { return row * 128 + ((ch ^ swz(row)) << 4); }
 
 // ---- STRIDED tile: 64 c-rows x R rows-of-the-operand; R*2-byte c-rows; chunk position =
