@@ -38,6 +38,9 @@ enum {
 };
 
 constexpr int BK = 64;  // contraction step, elements
+#ifndef OM_ROT_MODE
+#define OM_ROT_MODE 1
+#endif
 constexpr int NUM_XCD = 8;
 
 struct GemmParams {
@@ -187,6 +190,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     int expert, row_begin, row_end;  // fwd/dgrad: rows of this tile's expert segment
     int n0;                          // first output column (LDS B row 0)
     int c_begin, c_len;              // contraction range
+    int rot_a, rot_b;                // position among the tiles sharing this tile's A / B operand
     if (EPI == EPI_WGRAD) {
         // grid: x = (N/BM) * (K/BN) tiles of dW[g], y = expert; remapped so that an XCD works on
         // whole experts (all tiles of dW[g] share the expert's rows of both operands)
@@ -196,6 +200,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         expert = logical / tiles_e;
         const int tile = logical - expert * tiles_e;
         const int tm = tile / tiles_n, tn = tile % tiles_n;
+        rot_a = tn; rot_b = tm;
         row_begin = tm * BM;  // row of dW
         row_end = 0;
         n0 = tn * BN;
@@ -207,12 +212,25 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         const int logical = xcd_remap(blockIdx.x, gridDim.x);
         const int tile_m = logical / tiles_n;
         const int tile_n = logical % tiles_n;
+        rot_a = tile_n; rot_b = tile_m & 7;
         if (!find_tile<BM>(p.cum, p.n_experts, tile_m, lane, expert, row_begin, row_end)) return;
         n0 = tile_n * BN_OUT;
         c_begin = 0;
         c_len = p.kc;
     }
     const int steps_per_phase = (c_len + BK - 1) / BK;
+#if OM_ROT_MODE
+    // Tiles that run together on an XCD share operand slices.  Walking the contraction index from
+    // 0 in all of them makes them ask L2 for the same lines at the same time, and all wait for the
+    // same fill; a small per-tile offset lets one tile fetch a slice and the sharers hit it later.
+    const int rot = ((OM_ROT_MODE == 1 ? rot_a : (rot_a >> 1)) + rot_b) % (steps_per_phase > 0 ? steps_per_phase : 1);
+#else
+    const int rot = 0;
+#endif
+    auto rotated = [&](int sp) {   // sp in [0, steps_per_phase)
+        const int r = sp + rot;
+        return r >= steps_per_phase ? r - steps_per_phase : r;
+    };
     const int total_steps = steps_per_phase * p.phases;
 
     // ---- per-lane source offsets of the direct loads (elements, without the c0 term) ------------
@@ -272,7 +290,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     const int lda32 = static_cast<int>(p.lda), ldb32 = static_cast<int>(p.ldb);
     auto issue_loads = [&](int step, char *stage) {
         const int ph = (step >= steps_per_phase) ? 1 : 0;  // at most two phases
-        int c0 = (step - ph * steps_per_phase) * BK;
+        const int sp = step - ph * steps_per_phase;
+        int c0 = (sp < steps_per_phase ? rotated(sp) : sp) * BK;   // padding steps stay past the end
         if (EPI != EPI_WGRAD && c0 > c_len - BK) c0 = c_len - BK;
         const char *Ap = reinterpret_cast<const char *>(p.phases > 1 && ph ? p.A[1] : p.A[0]);
         const char *Bp = reinterpret_cast<const char *>(
@@ -309,7 +328,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // before the barrier).  B holds finite in-segment data there, so the products vanish.
     auto zero_tail = [&](int step, char *stage) {
         if (EPI != EPI_WGRAD) return;
-        const int c0 = step * BK;
+        const int c0 = (step < steps_per_phase ? rotated(step) : step) * BK;
         if (c0 + BK <= c_len) return;
         char *sa = stage + wave * (A_LOADS * 1024);
 #pragma unroll
@@ -405,6 +424,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         if (TM * TN > DS_READS) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - DS_READS, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
+    // same, with the direct loads of the next step spread between the MFMAs instead of ahead of them
+    auto interleave_loads = [&]() {
+        constexpr int NL = A_LOADS + B_LOADS;
+        constexpr int NM = TM * TN;
+#pragma unroll
+        for (int r = 0; r < NM; r++) {
+            if (r < NL) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);        // 1 VMEM read
+            if (r < DS_READS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                    // 1 MFMA
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
     // one contraction step on `cur`; `nxt` holds step s+1 when this returns
     auto half_step = [&](char *cur, char *nxt, int s) {
 #pragma unroll
@@ -419,7 +450,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         issue_loads(s + 2, cur);             // past the end on the last steps: harmless re-read
         read_group(nxt, 0, 0);
         mfma_group((BK / 16 - 1) & 1);
-        interleave();
+        interleave_loads();
     };
     // Steps are taken in pairs so the stage names are static; an odd step count (wgrad only: the
     // host requires kc % 128 == 0 otherwise) is padded with a step whose A tile is all zero.
