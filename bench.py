@@ -182,7 +182,42 @@ def bench_adamw(args, device):
     kern_ms = [a.elapsed_time(b) for _, a, b in log]
     avg_s = sum(kern_ms) / len(kern_ms) * 1e-3
     gbs = 28.0 * n / avg_s / 1e9
-    del st
+
+    # The gradient-norm pass and the update with the clip folded in (optimizers.py:136-160 then
+    # :162-205): one plan over 54 equal "parameters", coefficient 1.0 so the data stay put.
+    from optimus.optimizers import GradNormPlan
+    n_par = 54
+    sizes = [n // n_par] * (n_par - 1) + [n - (n // n_par) * (n_par - 1)]
+    starts = [sum(sizes[:i]) for i in range(n_par)]
+    plan = GradNormPlan(starts, sizes, device)
+    one = torch.ones(1, dtype=torch.float32, device=device)
+
+    def timed(fn, names, reps=5):
+        fn(); fn()
+        torch.cuda.synchronize()
+        _native.launch_log = []
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        lg, _native.launch_log = _native.launch_log, None
+        return sum(a.elapsed_time(b) for nm, a, b in lg if nm in names) / reps * 1e-3
+
+    t_norm = timed(lambda: plan.run(st["grad"]), ("om_grad_sumsq", "om_grad_norm_clip_coef"))
+    t_clip = {}
+    for store in (True, False):
+        t_clip[store] = timed(lambda: adamw_step_(
+            st["param"], st["grad"], st["master"], st["exp_avg"], st["exp_avg_sq"], hp["step_id"] + 1,
+            hp["lr"], hp["betas"][0], hp["betas"][1], hp["eps"], hp["weight_decay"], grad_scale=one,
+            store_scaled_grad=store), ("om_adamw_step_clipped",))
+    grad_clip = {
+        "grad_norm_ms": round(t_norm * 1e3, 3), "grad_norm_gb_per_s": round(2.0 * n / t_norm / 1e9, 1),
+        "clipped_step_ms": round(t_clip[True] * 1e3, 3),
+        "clipped_step_gb_per_s": round(30.0 * n / t_clip[True] / 1e9, 1),
+        "clipped_step_no_store_ms": round(t_clip[False] * 1e3, 3),
+        "clipped_step_no_store_gb_per_s": round(28.0 * n / t_clip[False] / 1e9, 1),
+        "note": "norm pass reads 2 B/param; clipped step = 28 B/param + 2 B/param when the scaled "
+                "gradient is stored back; 54 parameter slices, 65536-element chunks"}
+    del st, plan
     torch.cuda.empty_cache()
     return {"metric": "adamw_step_hbm_gb_per_s", "value": round(gbs, 1), "unit": "GB/s",
             "ms_per_step": round((t1 - t0) * 1e3 / steps, 3), "steps": steps, "dtype": "f32",
@@ -190,7 +225,8 @@ def bench_adamw(args, device):
                                    "param/grad + fp32 master/m/v, step 100"},
             "roofline": {"bound": "hbm", "kernel": "om_adamw_step", "achieved": round(gbs, 1),
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
-                         "traffic": MEASURED_TRAFFIC_BYTES["om_adamw_step"], "bytes_per_param": 28, "kernel_avg_ms": round(avg_s * 1e3, 3)}}
+                         "traffic": MEASURED_TRAFFIC_BYTES["om_adamw_step"], "bytes_per_param": 28, "kernel_avg_ms": round(avg_s * 1e3, 3)},
+            "grad_clip": grad_clip}
 
 
 def cpu_baseline_adamw():

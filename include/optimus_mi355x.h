@@ -64,6 +64,40 @@ int om_adamw_step(void *param, const void *grad, float *master, float *exp_avg,
                   void *stream);
 
 /* ------------------------------------------------------------------------------------
+ * Gradient norm and clip coefficient over the flat gradient buffer
+ * replaces: the "4opt-step_grad-clip" block of MixedPrecisionAdamW.step,
+ *           optimus/optimizers.py:136-160 — torch.nn.utils.get_total_norm (always) and
+ *           clip_grad_norm_ / clip_grads_with_norm_ (max_norm 1.0, after warm-up) over the
+ *           parameters' gradient views (optimizers.py:109-111 makes them slices of flat_grad).
+ * The flat buffer is cut into chunks [chunk_offsets[c], chunk_offsets[c+1]) that never straddle
+ * two parameters; parameter s owns chunks [seg_first_chunk[s], seg_first_chunk[s+1]).  Both
+ * tables are int64 device arrays built once by the caller (any chunk length; 65536 elements is
+ * a good one).
+ * om_grad_sumsq: partials[c] = fp32 sum of squares of chunk c (one read of the gradients).
+ * om_grad_norm_clip_coef: seg_norms[s] = sqrt(sum of its partials) rounded to the gradient
+ *   dtype (what vector_norm returns for a bf16 tensor); *total_norm = norm of seg_norms, rounded
+ *   likewise; if clip_coef is not null, *clip_coef = min(1, max_norm * (1/(total_norm + 1e-6)))
+ *   with each intermediate rounded to the gradient dtype (torch evaluates the expression on a
+ *   0-dim tensor of that dtype).  All outputs are fp32 device scalars/arrays holding those
+ *   rounded values.                                                                       */
+int om_grad_sumsq(const void *grad, int grad_dtype, const int64_t *chunk_offsets,
+                  int64_t n_chunks, float *partials, void *stream);
+int om_grad_norm_clip_coef(const float *partials, const int64_t *seg_first_chunk,
+                           int64_t n_segs, int grad_dtype, double max_norm, float *seg_norms,
+                           float *total_norm, float *clip_coef, void *stream);
+
+/* om_adamw_step with the clip folded in: g = cast(grad * *grad_scale) is what the update uses,
+ * i.e. the in-place multiply of clip_grads_with_norm_ (optimizers.py:145/150/154) without its
+ * read-modify-write pass over the gradients.  *grad_scale is a device fp32 scalar (the clip_coef
+ * above).  store_scaled_grad != 0 also writes g back into `grad`, which leaves the gradient
+ * buffer as the reference leaves it (+2 B/element of traffic in bf16 mode); 0 leaves `grad`
+ * untouched.                                                                              */
+int om_adamw_step_clipped(void *param, void *grad, float *master, float *exp_avg,
+                          float *exp_avg_sq, int64_t n, double lr, double beta1, double beta2,
+                          double eps, double weight_decay, int64_t step, int param_dtype,
+                          const float *grad_scale, int store_scaled_grad, void *stream);
+
+/* ------------------------------------------------------------------------------------
  * Routers
  * om_route_softmax_topk replaces optimus/models/common/moe.py:467-471
  *   (= optimus/models/olmoe/modeling_olmoe.py:295-299): fp32 softmax over N experts,

@@ -34,21 +34,32 @@ __device__ __forceinline__ void adam_update(float g, float &m, float &v, float &
 #ifndef OM_ADAMW_UNROLL
 #define OM_ADAMW_UNROLL 4
 #endif
-template <int UNROLL>
+//
+// CLIP selects what happens to the gradient before the update (reference optimizers.py:136-152,
+// torch.nn.utils.clip_grads_with_norm_): 0 = used as is; 1 = multiplied by *grad_scale and rounded
+// back to the gradient dtype, as the in-place multiply of the bf16 gradient views does; 2 = the
+// same, and the scaled gradient is also stored (then `grad` is null and `grad_rw` is both the
+// source and the destination).
+template <int UNROLL, int CLIP>
 __global__ __launch_bounds__(256) void adamw_bf16_kernel(uint16_t *__restrict__ param,
                                                             const uint16_t *__restrict__ grad,
+                                                            uint16_t *grad_rw,
+                                                            const float *__restrict__ grad_scale,
                                                             float *__restrict__ master,
                                                             float *__restrict__ exp_avg,
                                                             float *__restrict__ exp_avg_sq,
                                                             int64_t n_vec4, AdamScalars s) {
     const int64_t base = (static_cast<int64_t>(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
+    const uint16_t *gsrc = CLIP == 2 ? grad_rw : grad;
+    float coef = 1.0f;
+    if (CLIP) coef = *grad_scale;
     u32x2 gq[UNROLL];
     f32x4 m0[UNROLL], v0[UNROLL], w0[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
         const int64_t c = base + static_cast<int64_t>(u) * 256;
         if (c < n_vec4) {
-            gq[u] = *(reinterpret_cast<const u32x2 *>(grad) + c);
+            gq[u] = *(reinterpret_cast<const u32x2 *>(gsrc) + c);
             m0[u] = *(reinterpret_cast<const f32x4 *>(exp_avg) + c);
             v0[u] = *(reinterpret_cast<const f32x4 *>(exp_avg_sq) + c);
             w0[u] = *(reinterpret_cast<const f32x4 *>(master) + c);
@@ -63,6 +74,20 @@ __global__ __launch_bounds__(256) void adamw_bf16_kernel(uint16_t *__restrict__ 
             g[1] = __uint_as_float(gq[u][0] & 0xffff0000u);
             g[2] = __uint_as_float(gq[u][1] << 16);
             g[3] = __uint_as_float(gq[u][1] & 0xffff0000u);
+            if (CLIP) {
+                uint16_t gb[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    gb[i] = f32_to_bf16_bits(g[i] * coef);
+                    g[i] = bf16_bits_to_f32(gb[i]);
+                }
+                if (CLIP == 2) {
+                    u32x2 gs;
+                    gs[0] = static_cast<uint32_t>(gb[0]) | (static_cast<uint32_t>(gb[1]) << 16);
+                    gs[1] = static_cast<uint32_t>(gb[2]) | (static_cast<uint32_t>(gb[3]) << 16);
+                    *(reinterpret_cast<u32x2 *>(grad_rw) + c) = gs;
+                }
+            }
             float w[4];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -83,31 +108,47 @@ __global__ __launch_bounds__(256) void adamw_bf16_kernel(uint16_t *__restrict__ 
 }
 
 // Elements past the last full vector of 4 (at most 3).
-__global__ void adamw_bf16_tail_kernel(uint16_t *param, const uint16_t *grad, float *master,
-                                       float *exp_avg, float *exp_avg_sq, int64_t start, int64_t n,
-                                       AdamScalars s) {
+__global__ void adamw_bf16_tail_kernel(uint16_t *param, uint16_t *grad, const float *grad_scale,
+                                       int store_grad, float *master, float *exp_avg,
+                                       float *exp_avg_sq, int64_t start, int64_t n, AdamScalars s) {
     const int64_t i = start + threadIdx.x;
     if (i < n) {
         float m = exp_avg[i], v = exp_avg_sq[i], w = master[i];
-        adam_update(bf16_bits_to_f32(grad[i]), m, v, w, s);
+        float g = bf16_bits_to_f32(grad[i]);
+        if (grad_scale) {
+            const uint16_t gb = f32_to_bf16_bits(g * *grad_scale);
+            g = bf16_bits_to_f32(gb);
+            if (store_grad) grad[i] = gb;
+        }
+        adam_update(g, m, v, w, s);
         exp_avg[i] = m; exp_avg_sq[i] = v; master[i] = w;
         param[i] = f32_to_bf16_bits(w);
     }
 }
 
 // fp32 mode: the parameter buffer is the master buffer (16 B read, 12 B written per element).
-template <int UNROLL>
+template <int UNROLL, int CLIP>
 __global__ __launch_bounds__(256) void adamw_f32_kernel(float *__restrict__ master,
                                                         const float *__restrict__ grad,
+                                                        float *grad_rw,
+                                                        const float *__restrict__ grad_scale,
                                                         float *__restrict__ exp_avg,
                                                         float *__restrict__ exp_avg_sq,
                                                         int64_t n_vec4, AdamScalars s) {
     const int64_t base = (static_cast<int64_t>(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
+    const float *gsrc = CLIP == 2 ? grad_rw : grad;
+    float coef = 1.0f;
+    if (CLIP) coef = *grad_scale;
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
         const int64_t c = base + static_cast<int64_t>(u) * 256;
         if (c < n_vec4) {
-            f32x4 g = *(reinterpret_cast<const f32x4 *>(grad) + c);
+            f32x4 g = *(reinterpret_cast<const f32x4 *>(gsrc) + c);
+            if (CLIP) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) g[i] = g[i] * coef;
+                if (CLIP == 2) *(reinterpret_cast<f32x4 *>(grad_rw) + c) = g;
+            }
             f32x4 m = *(reinterpret_cast<const f32x4 *>(exp_avg) + c);
             f32x4 v = *(reinterpret_cast<const f32x4 *>(exp_avg_sq) + c);
             f32x4 w = *(reinterpret_cast<const f32x4 *>(master) + c);
@@ -123,27 +164,35 @@ __global__ __launch_bounds__(256) void adamw_f32_kernel(float *__restrict__ mast
         }
     }
 }
-__global__ void adamw_f32_tail_kernel(float *master, const float *grad, float *exp_avg,
-                                      float *exp_avg_sq, int64_t start, int64_t n, AdamScalars s) {
+__global__ void adamw_f32_tail_kernel(float *master, float *grad, const float *grad_scale,
+                                      int store_grad, float *exp_avg, float *exp_avg_sq,
+                                      int64_t start, int64_t n, AdamScalars s) {
     const int64_t i = start + threadIdx.x;
     if (i < n) {
         float m = exp_avg[i], v = exp_avg_sq[i], w = master[i];
-        adam_update(grad[i], m, v, w, s);
+        float g = grad[i];
+        if (grad_scale) {
+            g = g * *grad_scale;
+            if (store_grad) grad[i] = g;
+        }
+        adam_update(g, m, v, w, s);
         exp_avg[i] = m; exp_avg_sq[i] = v; master[i] = w;
     }
 }
 
 }  // namespace
 
-extern "C" int om_adamw_step(void *param, const void *grad, float *master, float *exp_avg,
-                             float *exp_avg_sq, int64_t n, double lr, double beta1, double beta2,
-                             double eps, double weight_decay, int64_t step, int param_dtype,
-                             void *stream) {
+// clip: 0 = gradient used as is, 1 = scaled by *grad_scale, 2 = scaled and stored back.
+static int adamw_launch(void *param, void *grad, float *master, float *exp_avg, float *exp_avg_sq,
+                        int64_t n, double lr, double beta1, double beta2, double eps,
+                        double weight_decay, int64_t step, int param_dtype, const float *grad_scale,
+                        int clip, void *stream) {
     if (param_dtype != OM_BF16 && param_dtype != OM_F32) return OM_ERR_DTYPE;
     if (n < 0 || step < 1) return OM_ERR_SHAPE;
     if (n == 0) return OM_OK;
     if (!grad || !master || !exp_avg || !exp_avg_sq) return OM_ERR_NULL;
     if (param_dtype == OM_BF16 && !param) return OM_ERR_NULL;
+    if (clip && !grad_scale) return OM_ERR_NULL;
     if (!om_aligned16(grad) || !om_aligned16(master) || !om_aligned16(exp_avg) ||
         !om_aligned16(exp_avg_sq) || (param_dtype == OM_BF16 && !om_aligned16(param)))
         return OM_ERR_ALIGN;
@@ -164,30 +213,61 @@ extern "C" int om_adamw_step(void *param, const void *grad, float *master, float
 
     hipStream_t st = om_stream(stream);
     constexpr int UNROLL = OM_ADAMW_UNROLL;
+    const int64_t n_vec = n / 4;
+    const int64_t blocks = (n_vec + 256 * UNROLL - 1) / (256 * UNROLL);
+    if (blocks > 0x7fffffffLL) return OM_ERR_SHAPE;
+    const dim3 grid(static_cast<unsigned>(blocks)), block(256);
     if (param_dtype == OM_BF16) {
-        const int64_t n_vec = n / 4;
+        uint16_t *p = static_cast<uint16_t *>(param), *g = static_cast<uint16_t *>(grad);
         if (n_vec > 0) {
-            const int64_t blocks = (n_vec + 256 * UNROLL - 1) / (256 * UNROLL);
-            if (blocks > 0x7fffffffLL) return OM_ERR_SHAPE;
-            adamw_bf16_kernel<UNROLL><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(
-                static_cast<uint16_t *>(param), static_cast<const uint16_t *>(grad), master, exp_avg,
-                exp_avg_sq, n_vec, s);
+            if (clip == 0)
+                adamw_bf16_kernel<UNROLL, 0><<<grid, block, 0, st>>>(p, g, nullptr, nullptr, master,
+                                                                     exp_avg, exp_avg_sq, n_vec, s);
+            else if (clip == 1)
+                adamw_bf16_kernel<UNROLL, 1><<<grid, block, 0, st>>>(p, g, nullptr, grad_scale, master,
+                                                                     exp_avg, exp_avg_sq, n_vec, s);
+            else
+                adamw_bf16_kernel<UNROLL, 2><<<grid, block, 0, st>>>(p, nullptr, g, grad_scale, master,
+                                                                     exp_avg, exp_avg_sq, n_vec, s);
         }
         if (n_vec * 4 < n)
-            adamw_bf16_tail_kernel<<<1, 64, 0, st>>>(static_cast<uint16_t *>(param),
-                                                     static_cast<const uint16_t *>(grad), master,
-                                                     exp_avg, exp_avg_sq, n_vec * 4, n, s);
+            adamw_bf16_tail_kernel<<<1, 64, 0, st>>>(p, g, clip ? grad_scale : nullptr, clip == 2,
+                                                     master, exp_avg, exp_avg_sq, n_vec * 4, n, s);
     } else {
-        const int64_t n_vec = n / 4;
+        float *g = static_cast<float *>(grad);
         if (n_vec > 0) {
-            const int64_t blocks = (n_vec + 256 * UNROLL - 1) / (256 * UNROLL);
-            if (blocks > 0x7fffffffLL) return OM_ERR_SHAPE;
-            adamw_f32_kernel<UNROLL><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(
-                master, static_cast<const float *>(grad), exp_avg, exp_avg_sq, n_vec, s);
+            if (clip == 0)
+                adamw_f32_kernel<UNROLL, 0><<<grid, block, 0, st>>>(master, g, nullptr, nullptr, exp_avg,
+                                                                    exp_avg_sq, n_vec, s);
+            else if (clip == 1)
+                adamw_f32_kernel<UNROLL, 1><<<grid, block, 0, st>>>(master, g, nullptr, grad_scale,
+                                                                    exp_avg, exp_avg_sq, n_vec, s);
+            else
+                adamw_f32_kernel<UNROLL, 2><<<grid, block, 0, st>>>(master, nullptr, g, grad_scale,
+                                                                    exp_avg, exp_avg_sq, n_vec, s);
         }
         if (n_vec * 4 < n)
-            adamw_f32_tail_kernel<<<1, 64, 0, st>>>(master, static_cast<const float *>(grad),
+            adamw_f32_tail_kernel<<<1, 64, 0, st>>>(master, g, clip ? grad_scale : nullptr, clip == 2,
                                                     exp_avg, exp_avg_sq, n_vec * 4, n, s);
     }
     return om_launch_status();
+}
+
+extern "C" int om_adamw_step(void *param, const void *grad, float *master, float *exp_avg,
+                             float *exp_avg_sq, int64_t n, double lr, double beta1, double beta2,
+                             double eps, double weight_decay, int64_t step, int param_dtype,
+                             void *stream) {
+    return adamw_launch(param, const_cast<void *>(grad), master, exp_avg, exp_avg_sq, n, lr, beta1,
+                        beta2, eps, weight_decay, step, param_dtype, nullptr, 0, stream);
+}
+
+extern "C" int om_adamw_step_clipped(void *param, void *grad, float *master, float *exp_avg,
+                                     float *exp_avg_sq, int64_t n, double lr, double beta1,
+                                     double beta2, double eps, double weight_decay, int64_t step,
+                                     int param_dtype, const float *grad_scale, int store_scaled_grad,
+                                     void *stream) {
+    if (!grad_scale) return OM_ERR_NULL;
+    return adamw_launch(param, grad, master, exp_avg, exp_avg_sq, n, lr, beta1, beta2, eps,
+                        weight_decay, step, param_dtype, grad_scale, store_scaled_grad ? 2 : 1,
+                        stream);
 }

@@ -116,28 +116,41 @@ class MixedPrecisionAdamW(Optimizer):
             if self.dtype != torch.float32 and (not self.skip_optimizer_step):
                 self.flat_fp32_master_param[start_ind:end_ind].view_as(p.data).copy_(p.data)
 
+        # Gradient-norm kernels run over flat_grad when it holds every gradient of the model
+        # (the reference takes the norm over model.parameters(), optimizers.py:143-158)
+        self.opt_store_clipped_grads = True   # leave flat_grad clipped after step(), as the reference does
+        owned = {id(p) for p in self.param_list}
+        model_params = list(self.model.parameters()) if self.model is not None else self.param_list
+        if self.flat_param_size > 0 and len(model_params) == len(owned) \
+                and all(id(p) in owned for p in model_params):
+            self._norm_plan = GradNormPlan(self.param_start_inds, self.param_sizes, self.device)
+        else:
+            self._norm_plan = None
+
     def zero_grad(self):
         self.flat_grad.zero_()
 
     def _grad_norm_and_clip(self):
-        """Gradient norm (always) and clip to 1.0 (after warm-up), reference optimizers.py:136-160.
-        Same torch.nn.utils calls as the reference, on the same parameter views."""
+        """Gradient norm (always) and the clip to 1.0 (after warm-up), reference
+        optimizers.py:136-160.  Returns (grad_norm, clip_coef): grad_norm is a 0-dim tensor in the
+        gradient dtype like torch.nn.utils.get_total_norm gives; clip_coef is a device fp32 scalar
+        for the update kernel to apply, or None when this step does not clip.  The single-step
+        and two-step variants of the reference compute the same thing on one device."""
         clip_now = self.opt_disable_delayed_grad_clipping or (self.step_id >= self.warmup_steps)
-        if clip_now:
-            if not self.opt_use_two_step_grad_clipping:
-                grad_norm = torch.nn.utils.clip_grad_norm_(self.model.parameters(), 1.0)
-            else:
-                grad_norm = torch.nn.utils.get_total_norm(
-                    [p.grad for p in self.model.parameters() if p.grad is not None])
+        if self._norm_plan is None:
+            # the model holds parameters this optimizer does not own: their gradients are not in
+            # flat_grad, so take the norm over the model's list with the library calls
+            grads = [p.grad for p in self.model.parameters() if p.grad is not None]
+            grad_norm = torch.nn.utils.get_total_norm(grads)
+            if clip_now:
                 torch.nn.utils.clip_grads_with_norm_(self.model.parameters(), 1.0, grad_norm)
-        else:
-            grad_norm = torch.nn.utils.get_total_norm(
-                [p.grad for p in self.model.parameters() if p.grad is not None])
-        return grad_norm
+            return grad_norm, None
+        total, coef = self._norm_plan.run(self.flat_grad, max_norm=1.0)
+        return total.to(self.flat_grad.dtype), (coef if clip_now else None)
 
     def step(self, closure=None):
         with record_pcl_function("4opt-step_grad-clip"):
-            grad_norm = self._grad_norm_and_clip()
+            grad_norm, clip_coef = self._grad_norm_and_clip()
 
         with record_pcl_function("4opt-step_compute"):
             if not self.skip_optimizer_step:
@@ -147,7 +160,11 @@ class MixedPrecisionAdamW(Optimizer):
                 weight_decay = self.defaults["weight_decay"]
                 adamw_step_(self.flat_param, self.flat_grad, self.flat_fp32_master_param,
                             self.flat_exp_avg, self.flat_exp_avg_sq, self.step_id + 1, lr, beta1,
-                            beta2, eps, weight_decay)
+                            beta2, eps, weight_decay, grad_scale=clip_coef,
+                            store_scaled_grad=self.opt_store_clipped_grads)
+            elif clip_coef is not None:
+                # no update kernel to fold the clip into
+                self.flat_grad.mul_(clip_coef.to(self.flat_grad.dtype))
         # Update step
         self.step_id += 1
 
@@ -170,9 +187,11 @@ class MixedPrecisionAdamW(Optimizer):
 
 
 def adamw_step_(flat_param, flat_grad, flat_master, flat_exp_avg, flat_exp_avg_sq, step, lr, beta1,
-                beta2, eps, weight_decay):
+                beta2, eps, weight_decay, grad_scale=None, store_scaled_grad=True):
     """One AdamW update over flat buffers, in place (the reference's compute block,
-    optimus/optimizers.py:162-205, as a single HIP pass).  `step` is 1-based (step_id + 1)."""
+    optimus/optimizers.py:162-205, as a single HIP pass).  `step` is 1-based (step_id + 1).
+    `grad_scale` (device fp32 scalar) folds the gradient clip in: the update uses
+    cast(grad * grad_scale), and stores it back into flat_grad if `store_scaled_grad`."""
     _n.require_cuda_contiguous(flat_param, flat_grad, flat_master, flat_exp_avg, flat_exp_avg_sq)
     n = flat_master.numel()
     if flat_grad.numel() != n or flat_exp_avg.numel() != n or flat_exp_avg_sq.numel() != n \
@@ -190,7 +209,61 @@ def adamw_step_(flat_param, flat_grad, flat_master, flat_exp_avg, flat_exp_avg_s
         code = _n.OM_BF16
     else:
         raise TypeError("flat_param / flat_grad must both be bfloat16 or both float32")
-    _n.check(_n.lib().om_adamw_step(_n.ptr(flat_param), _n.ptr(flat_grad), _n.ptr(flat_master),
-                                    _n.ptr(flat_exp_avg), _n.ptr(flat_exp_avg_sq), n, float(lr),
-                                    float(beta1), float(beta2), float(eps), float(weight_decay),
-                                    int(step), code, _n.stream()), "om_adamw_step")
+    args = (_n.ptr(flat_param), _n.ptr(flat_grad), _n.ptr(flat_master), _n.ptr(flat_exp_avg),
+            _n.ptr(flat_exp_avg_sq), n, float(lr), float(beta1), float(beta2), float(eps),
+            float(weight_decay), int(step), code)
+    if grad_scale is None:
+        _n.check(_n.lib().om_adamw_step(*args, _n.stream()), "om_adamw_step")
+    else:
+        _n.require_cuda_contiguous(grad_scale)
+        if grad_scale.dtype != torch.float32 or grad_scale.numel() != 1:
+            raise TypeError("grad_scale must be one float32 element on the device")
+        _n.check(_n.lib().om_adamw_step_clipped(*args, _n.ptr(grad_scale), int(bool(store_scaled_grad)),
+                                                _n.stream()), "om_adamw_step_clipped")
+
+
+class GradNormPlan:
+    """Chunk tables and scratch for the gradient-norm kernels over one flat gradient buffer.
+
+    `starts[i]`, `sizes[i]` give parameter i's slice of the flat buffer (reference
+    optimizers.py:86-92 `param_start_inds`, `param_sizes`).  The norm of every slice, the norm of
+    those norms and the clip coefficient come out as torch.nn.utils.get_total_norm and
+    clip_grads_with_norm_ compute them, including the roundings to the gradient dtype."""
+
+    CHUNK = 1 << 16
+
+    def __init__(self, starts, sizes, device, chunk=None):
+        chunk = int(chunk or self.CHUNK)
+        if len(sizes) == 0 or len(starts) != len(sizes):
+            raise ValueError("GradNormPlan needs one (start, size) pair per parameter")
+        begins, first, pos = [], [0], int(starts[0])
+        for st, sz in zip(starts, sizes):
+            st, sz = int(st), int(sz)
+            if st != pos:
+                raise ValueError("GradNormPlan: parameter slices must tile the flat buffer in order, "
+                                 "without gaps")
+            begins.append(torch.arange(st, st + sz, chunk, dtype=torch.int64))
+            first.append(first[-1] + (sz + chunk - 1) // chunk)
+            pos = st + sz
+        table = torch.cat(begins + [torch.tensor([pos], dtype=torch.int64)])
+        self.n_chunks = first[-1]
+        self.n_segs = len(sizes)
+        self.chunk_offsets = table.to(device)
+        self.seg_first_chunk = torch.tensor(first, dtype=torch.int64).to(device)
+        self.partials = torch.empty(max(self.n_chunks, 1), dtype=torch.float32, device=device)
+        self.seg_norms = torch.empty(self.n_segs, dtype=torch.float32, device=device)
+        self.out = torch.empty(2, dtype=torch.float32, device=device)   # total norm, clip coef
+
+    def run(self, flat_grad, max_norm=1.0):
+        """Returns (total_norm, clip_coef) as 0-dim float32 device tensors (views of one buffer
+        that the next call overwrites)."""
+        _n.require_cuda_contiguous(flat_grad)
+        code = _n.dtype_code(flat_grad)
+        lib = _n.lib()
+        _n.check(lib.om_grad_sumsq(_n.ptr(flat_grad), code, _n.ptr(self.chunk_offsets), self.n_chunks,
+                                   _n.ptr(self.partials), _n.stream()), "om_grad_sumsq")
+        _n.check(lib.om_grad_norm_clip_coef(_n.ptr(self.partials), _n.ptr(self.seg_first_chunk),
+                                            self.n_segs, code, float(max_norm), _n.ptr(self.seg_norms),
+                                            _n.ptr(self.out), _n.ptr(self.out) + 4, _n.stream()),
+                 "om_grad_norm_clip_coef")
+        return self.out[0], self.out[1:2]

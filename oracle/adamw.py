@@ -31,3 +31,17 @@ def adamw_step_torch(flat_param, flat_grad, flat_master, flat_exp_avg, flat_exp_
         if weight_decay > 0.0:
             master.add_(master, alpha=(-lr * weight_decay))                      # :202
         data.copy_(master.to(data.dtype))                                        # :205
+
+
+def grad_norm_and_clip_torch(grads, clip, max_norm=1.0):
+    """The reference's gradient-norm block for one device, optimus/optimizers.py:136-160: the
+    norm is always taken (`get_total_norm`), the clip (`clip_grads_with_norm_`, equivalently
+    `clip_grad_norm_`) only when `clip`.  `grads` are CPU tensors, scaled in place.  These are
+    the library calls the reference makes, so this is the pin for the scalar C restatement."""
+    total = torch.nn.utils.get_total_norm(grads)                                  # :147/:156
+    if clip:
+        holders = [torch.nn.Parameter(torch.empty_like(g)) for g in grads]
+        for h, g in zip(holders, grads):
+            h.grad = g
+        torch.nn.utils.clip_grads_with_norm_(holders, max_norm, total)           # :148
+    return total

@@ -107,3 +107,69 @@ void orc_adamw_step_f64(const bf16_t *grad, double *master, double *exp_avg,
         exp_avg[i] = m; exp_avg_sq[i] = v; master[i] = w;
     }
 }
+
+/*
+ * Gradient norm and clip, optimizers.py:136-160: torch.nn.utils.get_total_norm over the
+ * parameters' gradient views, then clip_grads_with_norm_(max_norm) when the step clips.
+ * What those library calls compute for bf16 gradients (fp32 arithmetic inside each op, the
+ * result of each op rounded to the tensor dtype):
+ *   norm_i = bf16( sqrt( sum_j g_ij^2 ) )                 vector_norm of one gradient
+ *   total  = bf16( sqrt( sum_i norm_i^2 ) )               vector_norm of the stacked norms
+ *   coef   = min( bf16( bf16( 1 / bf16(total + 1e-6) ) * max_norm ), 1 )
+ *            (max_norm / tensor is evaluated as tensor.reciprocal() * max_norm)
+ *   g_ij   = bf16( g_ij * coef )                          in-place multiply by the 0-dim tensor
+ * The sums are taken in double here and rounded once to float: the library's own summation order
+ * is not specified, and any fp32 order differs from this by far less than one bf16 step except
+ * exactly at a rounding boundary.
+ */
+void orc_grad_norm_clip_bf16(const bf16_t *grad, const int64_t *starts, const int64_t *sizes,
+                             int64_t n_params, double max_norm, float *seg_norms,
+                             float *total_norm, float *clip_coef) {
+    double tot = 0.0;
+    for (int64_t p = 0; p < n_params; p++) {
+        double acc = 0.0;
+        for (int64_t j = 0; j < sizes[p]; j++) {
+            double g = (double)bf16_to_f32(grad[starts[p] + j]);
+            acc += g * g;
+        }
+        float nrm = bf16_to_f32(f32_to_bf16(sqrtf((float)acc)));
+        seg_norms[p] = nrm;
+        tot += (double)nrm * (double)nrm;
+    }
+    float total = bf16_to_f32(f32_to_bf16(sqrtf((float)tot)));
+    *total_norm = total;
+    float x = bf16_to_f32(f32_to_bf16(total + 1e-6f));
+    float r = bf16_to_f32(f32_to_bf16(1.0f / x));
+    float c = bf16_to_f32(f32_to_bf16(r * (float)max_norm));
+    *clip_coef = c > 1.0f ? 1.0f : c;
+}
+
+void orc_grad_norm_clip_f32(const float *grad, const int64_t *starts, const int64_t *sizes,
+                            int64_t n_params, double max_norm, float *seg_norms,
+                            float *total_norm, float *clip_coef) {
+    double tot = 0.0;
+    for (int64_t p = 0; p < n_params; p++) {
+        double acc = 0.0;
+        for (int64_t j = 0; j < sizes[p]; j++) {
+            double g = (double)grad[starts[p] + j];
+            acc += g * g;
+        }
+        float nrm = sqrtf((float)acc);
+        seg_norms[p] = nrm;
+        tot += (double)nrm * (double)nrm;
+    }
+    float total = sqrtf((float)tot);
+    *total_norm = total;
+    float x = total + 1e-6f;
+    float r = 1.0f / x;
+    float c = r * (float)max_norm;
+    *clip_coef = c > 1.0f ? 1.0f : c;
+}
+
+/* The in-place multiply of clip_grads_with_norm_: g = cast(float(g) * coef). */
+void orc_scale_grads_bf16(bf16_t *grad, int64_t n, float coef) {
+    for (int64_t i = 0; i < n; i++) grad[i] = f32_to_bf16(bf16_to_f32(grad[i]) * coef);
+}
+void orc_scale_grads_f32(float *grad, int64_t n, float coef) {
+    for (int64_t i = 0; i < n; i++) grad[i] = grad[i] * coef;
+}

@@ -215,3 +215,24 @@ def adamw_step_f64(grad, master, exp_avg, exp_avg_sq, lr, beta1, beta2, eps, wei
     lib().orc_adamw_step_f64(_p(grad), _p(master), _p(exp_avg), _p(exp_avg_sq), I64(master.size),
                              F64(lr), F64(beta1), F64(beta2), F64(eps), F64(weight_decay),
                              I64(step))
+
+
+def grad_norm_clip(grad, starts, sizes, max_norm=1.0):
+    """Per-parameter norms, total norm and clip coefficient of a flat gradient buffer
+    (uint16 bf16 bits or float32).  Returns (seg_norms float32[P], total_norm, clip_coef)."""
+    assert grad.flags.c_contiguous and grad.dtype in (np.uint16, np.float32)
+    starts = np.ascontiguousarray(starts, dtype=np.int64)
+    sizes = np.ascontiguousarray(sizes, dtype=np.int64)
+    seg = np.zeros(len(sizes), dtype=np.float32)
+    total = np.zeros(1, dtype=np.float32)
+    coef = np.zeros(1, dtype=np.float32)
+    fn = lib().orc_grad_norm_clip_bf16 if grad.dtype == np.uint16 else lib().orc_grad_norm_clip_f32
+    fn(_p(grad), _p(starts), _p(sizes), I64(len(sizes)), F64(max_norm), _p(seg), _p(total), _p(coef))
+    return seg, float(total[0]), float(coef[0])
+
+
+def scale_grads(grad, coef):
+    """In place: grad = cast(float(grad) * coef)."""
+    assert grad.flags.c_contiguous and grad.dtype in (np.uint16, np.float32)
+    fn = lib().orc_scale_grads_bf16 if grad.dtype == np.uint16 else lib().orc_scale_grads_f32
+    fn(_p(grad), I64(grad.size), ctypes.c_float(coef))
