@@ -38,6 +38,13 @@ enum {
 };
 
 constexpr int BK = 64;  // contraction step, elements
+// shares (in eighths) of a step's direct loads issued after the barrier / with slices 0, 1, 2
+#ifndef OM_LD_T
+#define OM_LD_T 4
+#define OM_LD_0 4
+#define OM_LD_1 0
+#define OM_LD_2 0
+#endif
 #ifndef OM_ROT_MODE
 #define OM_ROT_MODE 1
 #endif
@@ -61,6 +68,8 @@ struct GemmParams {
     int kc;                     // contraction length per phase (fwd/dgrad), multiple of 64
     int phases;                 // 1 or 2
     int m_tiles_max;            // fwd/dgrad: upper bound on row tiles
+    int total_tiles;            // logical tiles of the launch (the blocks loop over them)
+    int tiles_e;                // wgrad: tiles per expert
 };
 
 typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_ptr;
@@ -158,14 +167,6 @@ __device__ __forceinline__ bool find_tile(const int32_t *cum, int n_experts, int
     return false;
 }
 
-// Give every XCD a contiguous run of logical tiles (hardware sends block b to XCD b % 8).
-__device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
-    const int per = nblocks / NUM_XCD;       // blocks in the evenly divisible part
-    const int body = per * NUM_XCD;
-    if (bid >= body) return bid;             // tail keeps its order
-    return (bid % NUM_XCD) * per + bid / NUM_XCD;
-}
-
 template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const GemmParams p) {
     constexpr int NW = WAVES_M * WAVES_N;
@@ -186,109 +187,132 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     const int wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-    // ---- which tile ---------------------------------------------------------------------
-    int expert, row_begin, row_end;  // fwd/dgrad: rows of this tile's expert segment
-    int n0;                          // first output column (LDS B row 0)
-    int c_begin, c_len;              // contraction range
-    int rot_a, rot_b;                // position among the tiles sharing this tile's A / B operand
-    if (EPI == EPI_WGRAD) {
-        // grid: x = (N/BM) * (K/BN) tiles of dW[g], y = expert; remapped so that an XCD works on
-        // whole experts (all tiles of dW[g] share the expert's rows of both operands)
-        const int tiles_n = p.n_cols / BN;
-        const int tiles_e = gridDim.x;
-        const int logical = xcd_remap(blockIdx.y * tiles_e + blockIdx.x, tiles_e * gridDim.y);
-        expert = logical / tiles_e;
-        const int tile = logical - expert * tiles_e;
-        const int tm = tile / tiles_n, tn = tile % tiles_n;
-        rot_a = tn; rot_b = tm;
-        row_begin = tm * BM;  // row of dW
-        row_end = 0;
-        n0 = tn * BN;
-        c_begin = p.cum[expert];
-        c_len = p.cum[expert + 1] - c_begin;
-    } else {
-        constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
-        const int tiles_n = p.n_cols / BN_OUT;
-        const int logical = xcd_remap(blockIdx.x, gridDim.x);
-        const int tile_m = logical / tiles_n;
-        const int tile_n = logical % tiles_n;
-        rot_a = tile_n; rot_b = tile_m & 7;
-        if (!find_tile<BM>(p.cum, p.n_experts, tile_m, lane, expert, row_begin, row_end)) return;
-        n0 = tile_n * BN_OUT;
-        c_begin = 0;
-        c_len = p.kc;
-    }
-    const int steps_per_phase = (c_len + BK - 1) / BK;
-#if OM_ROT_MODE
+    // ---- per-tile state (set by setup_tile) ---------------------------------------------------
+    int expert = 0, row_begin = 0, row_end = 0;  // fwd/dgrad: rows of this tile's expert segment
+    int n0 = 0;                                  // first output column (LDS B row 0)
+    int c_begin = 0, c_len = 0;                  // contraction range
+    int steps_per_phase = 0, total_steps = 0;
+    int loop_steps = 0;   // steps are taken in pairs: total_steps rounded up to even
     // Tiles that run together on an XCD share operand slices.  Walking the contraction index from
     // 0 in all of them makes them ask L2 for the same lines at the same time, and all wait for the
-    // same fill; a small per-tile offset lets one tile fetch a slice and the sharers hit it later.
-    const int rot = ((OM_ROT_MODE == 1 ? rot_a : (rot_a >> 1)) + rot_b) % (steps_per_phase > 0 ? steps_per_phase : 1);
-#else
-    const int rot = 0;
-#endif
+    // same fill; a small per-tile offset `rot` lets one tile fetch a slice and the sharers hit it.
+    int rot = 0;
     auto rotated = [&](int sp) {   // sp in [0, steps_per_phase)
         const int r = sp + rot;
         return r >= steps_per_phase ? r - steps_per_phase : r;
     };
-    const int total_steps = steps_per_phase * p.phases;
 
     // ---- per-lane source offsets of the direct loads (elements, without the c0 term) ------------
     // CONTIG : lane -> (row = group*8 + lane/8, chunk = (lane%8) ^ swz(row))
     // STRIDED: lane -> (crow = group*(64/CPR) + lane/CPR, chunk = (lane%CPR) ^ ((crow&3)<<2))
     int a_off[A_LOADS], b_off[B_LOADS];  // the host checks that every operand spans < 2^31 elements
     int a_crow[A_LOADS];  // STRIDED A in wgrad: c-row of the lane's slot (for the zero fill)
+    int b_crow[B_LOADS];
+    bool b_up[B_LOADS];   // EPI_SWIGLU: this LDS row comes from the up matrix
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
-        const int grp = wave * A_LOADS + i;
-        if (AKIND == CONTIG) {
-            const int row = grp * 8 + (lane >> 3);
-            const int ch = (lane & 7) ^ swz(row);
-            int64_t m = static_cast<int64_t>(row_begin) + row;
-            if (m >= row_end) m = row_end - 1;  // rows past the segment: valid memory, result unused
-            a_off[i] = static_cast<int>(m * p.lda + ch * 8);
-            a_crow[i] = 0;
-        } else {
-            constexpr int CPR = BM / 8;
-            const int crow = grp * (64 / CPR) + lane / CPR;
-            const int ch = (lane % CPR) ^ ((crow & 3) << 2);
-            a_off[i] = row_begin + ch * 8;  // + (c_begin + c) * lda per step
-            a_crow[i] = crow;
-        }
+        constexpr int CPR = BM / 8;
+        a_crow[i] = (AKIND == CONTIG) ? 0 : (wave * A_LOADS + i) * (64 / CPR) + lane / CPR;
     }
-    int b_crow[B_LOADS];
-    bool b_up[B_LOADS];  // EPI_SWIGLU: this LDS row comes from the up matrix
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
+        constexpr int CPR = BN / 8;
         const int grp = wave * B_LOADS + i;
-        if (BKIND == CONTIG) {
-            const int row = grp * 8 + (lane >> 3);
-            const int ch = (lane & 7) ^ swz(row);
-            if (EPI == EPI_SWIGLU) {
-                // LDS rows alternate 32 gate rows / 32 up rows; the up matrix is B[1]
-                const int blk = row >> 5;
-                const int64_t n = n0 + (blk >> 1) * 32 + (row & 31);
-                b_off[i] = static_cast<int>(expert * p.strideB + n * p.ldb + ch * 8);
-                b_up[i] = blk & 1;
-            } else {
-                b_off[i] = static_cast<int>(expert * p.strideB + static_cast<int64_t>(n0 + row) * p.ldb + ch * 8);
-            }
-            b_crow[i] = 0;
-            if (EPI != EPI_SWIGLU) b_up[i] = false;
-        } else {
-            b_up[i] = false;
-            constexpr int CPR = BN / 8;
-            const int crow = grp * (64 / CPR) + lane / CPR;
-            const int ch = (lane % CPR) ^ ((crow & 3) << 2);
-            b_off[i] = static_cast<int>((EPI == EPI_WGRAD ? 0 : expert * p.strideB) + n0 + ch * 8);
-            b_crow[i] = crow;
-        }
+        b_crow[i] = (BKIND == CONTIG) ? 0 : grp * (64 / CPR) + lane / CPR;
+        b_up[i] = (EPI == EPI_SWIGLU) ? (((grp * 8 + (lane >> 3)) >> 5) & 1) : false;
     }
 
-    // Loads of contraction step `step` into `stage`.  Steps past the end (the loop always works on
-    // pairs of steps) re-read the last valid slice; their data is never multiplied, or is zeroed.
+    // Which tile `logical` is, and the load offsets for it.  False: the tile lies past the last
+    // row block (the launch sizes the tile count from an upper bound on the routed rows).
+    auto setup_tile = [&](int logical) -> bool {
+        int rot_a, rot_b;  // position among the tiles sharing this tile's A / B operand
+        // lane-derived terms are recomputed per tile rather than kept live across the main loop
+        int lane_s = lane;
+        asm volatile("" : "+v"(lane_s));
+        if (EPI == EPI_WGRAD) {
+            // tiles are numbered expert-major: an XCD works on whole experts (all tiles of dW[g]
+            // share the expert's rows of both operands)
+            const int tiles_n = p.n_cols / BN;
+            expert = logical / p.tiles_e;
+            const int tile = logical - expert * p.tiles_e;
+            const int tm = tile / tiles_n, tn = tile % tiles_n;
+            rot_a = tn; rot_b = tm;
+            row_begin = tm * BM;  // row of dW
+            row_end = 0;
+            n0 = tn * BN;
+            c_begin = p.cum[expert];
+            c_len = p.cum[expert + 1] - c_begin;
+        } else {
+            constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
+            const int tiles_n = p.n_cols / BN_OUT;
+            const int tile_m = logical / tiles_n;
+            const int tile_n = logical % tiles_n;
+            rot_a = tile_n; rot_b = tile_m & 7;
+            if (!find_tile<BM>(p.cum, p.n_experts, tile_m, lane_s, expert, row_begin, row_end)) return false;
+            n0 = tile_n * BN_OUT;
+            c_begin = 0;
+            c_len = p.kc;
+        }
+        // block-uniform values: keep them in scalar registers
+        expert = __builtin_amdgcn_readfirstlane(expert);
+        row_begin = __builtin_amdgcn_readfirstlane(row_begin);
+        row_end = __builtin_amdgcn_readfirstlane(row_end);
+        n0 = __builtin_amdgcn_readfirstlane(n0);
+        c_begin = __builtin_amdgcn_readfirstlane(c_begin);
+        c_len = __builtin_amdgcn_readfirstlane(c_len);
+        steps_per_phase = (c_len + BK - 1) / BK;
+        total_steps = steps_per_phase * p.phases;
+        loop_steps = (total_steps + 1) & ~1;
+#if OM_ROT_MODE
+        rot = ((OM_ROT_MODE == 1 ? rot_a : (rot_a >> 1)) + rot_b) % (steps_per_phase > 0 ? steps_per_phase : 1);
+#else
+        rot = 0;
+#endif
+#pragma unroll
+        for (int i = 0; i < A_LOADS; i++) {
+            const int grp = wave * A_LOADS + i;
+            if (AKIND == CONTIG) {
+                const int row = grp * 8 + (lane_s >> 3);
+                const int ch = (lane_s & 7) ^ swz(row);
+                int64_t m = static_cast<int64_t>(row_begin) + row;
+                if (m >= row_end) m = row_end - 1;  // rows past the segment: valid memory, result unused
+                a_off[i] = static_cast<int>(m * p.lda + ch * 8);
+            } else {
+                constexpr int CPR = BM / 8;
+                const int ch = (lane_s % CPR) ^ ((a_crow[i] & 3) << 2);
+                a_off[i] = row_begin + ch * 8;  // + (c_begin + c) * lda per step
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; i++) {
+            const int grp = wave * B_LOADS + i;
+            if (BKIND == CONTIG) {
+                const int row = grp * 8 + (lane_s >> 3);
+                const int ch = (lane_s & 7) ^ swz(row);
+                if (EPI == EPI_SWIGLU) {
+                    // LDS rows alternate 32 gate rows / 32 up rows; the up matrix is B[1]
+                    const int blk = row >> 5;
+                    const int64_t n = n0 + (blk >> 1) * 32 + (row & 31);
+                    b_off[i] = static_cast<int>(expert * p.strideB + n * p.ldb + ch * 8);
+                } else {
+                    b_off[i] = static_cast<int>(expert * p.strideB + static_cast<int64_t>(n0 + row) * p.ldb + ch * 8);
+                }
+            } else {
+                constexpr int CPR = BN / 8;
+                const int ch = (lane_s % CPR) ^ ((b_crow[i] & 3) << 2);
+                b_off[i] = static_cast<int>((EPI == EPI_WGRAD ? 0 : expert * p.strideB) + n0 + ch * 8);
+            }
+        }
+        return true;
+    };
+
+    // Loads of contraction step `step` into `stage`.  The padding step of an odd step count (the
+    // loop works on pairs of steps) re-reads the last valid slice; its A tile is zeroed.
     const int lda32 = static_cast<int>(p.lda), ldb32 = static_cast<int>(p.ldb);
-    auto issue_loads = [&](int step, char *stage) {
+    // Loads [lo, hi) of the step's list (A loads first, then B loads); lo and hi are constants
+    // after unrolling.
+    auto issue_part = [&](int step, char *stage, int lo, int hi) {
+        if (step >= loop_steps) return;                    // nothing left to fetch for this tile
         const int ph = (step >= steps_per_phase) ? 1 : 0;  // at most two phases
         const int sp = step - ph * steps_per_phase;
         int c0 = (sp < steps_per_phase ? rotated(sp) : sp) * BK;   // padding steps stay past the end
@@ -301,6 +325,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         char *sb = stage + A_BYTES + wave * (B_LOADS * 1024);
 #pragma unroll
         for (int i = 0; i < A_LOADS; i++) {
+            if (i < lo || i >= hi) continue;
             uint32_t off;  // bytes from the operand base; < 2^32 (checked on the host)
             if (AKIND == CONTIG) {
                 off = static_cast<uint32_t>(a_off[i] + c0) * 2u;
@@ -313,6 +338,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         }
 #pragma unroll
         for (int i = 0; i < B_LOADS; i++) {
+            if (A_LOADS + i < lo || A_LOADS + i >= hi) continue;
             uint32_t off;
             if (BKIND == CONTIG) {
                 off = static_cast<uint32_t>(b_off[i] + c0) * 2u;
@@ -324,6 +350,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             load16_to_lds(((EPI == EPI_SWIGLU && b_up[i]) ? Bup : Bp) + off, sb + i * 1024);
         }
     };
+    constexpr int NL = A_LOADS + B_LOADS;
+    auto issue_loads = [&](int step, char *stage) { issue_part(step, stage, 0, NL); };
+    // The direct loads of a step are spread over the MFMAs of a whole step rather than issued in
+    // one burst: the texture path of a CU accepts about one 1 KB load per wavefront every ~220
+    // cycles, and a wavefront that has to wait for it cannot issue its MFMAs meanwhile.  Shares of
+    // the NL loads: after the barrier of step s (stage free), then with slices 0, 1, 2 of step s+1.
+    constexpr int LD_T = NL * OM_LD_T / 8, LD_0 = NL * OM_LD_0 / 8, LD_1 = NL * OM_LD_1 / 8;
+    constexpr int LD_2 = NL - LD_T - LD_0 - LD_1;
+    static_assert(OM_LD_T + OM_LD_0 + OM_LD_1 + OM_LD_2 == 8 && LD_2 >= 0, "load shares");
     // wgrad: zero the A c-rows past the end of the expert's rows (after the loads have landed,
     // before the barrier).  B holds finite in-segment data there, so the products vanish.
     auto zero_tail = [&](int step, char *stage) {
@@ -338,12 +373,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     };
 
     f32x16 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     // ---- fragment addresses (bytes within a stage), loop-invariant ------------------------------
     // CONTIG : addr(i, kk) = c_base + i*4096 + c_kofs[kk]      (rows i*32 apart share the swizzle)
@@ -413,61 +442,107 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                 // operands swapped: the lane then holds 4 consecutive output columns per row
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
     };
-    // scheduling hint: one LDS read, then one MFMA, ... then the remaining MFMAs
+    // Scheduling hint for one 16-slice: MFMA first, then the LDS reads of the next slice two at a
+    // time behind the leading MFMAs, `nl` direct loads spread evenly, the remaining MFMAs last.
+    // The wait for the previous slice's fragments then sits ahead of the first MFMA with no newer
+    // LDS read in front of it (the compiler always waits for a zero LDS counter here because the
+    // direct loads count as possible LDS accesses), and the last read of a slice has several MFMAs
+    // behind it to hide its latency.
     constexpr int DS_READS = TM * (AKIND == CONTIG ? 1 : 2) + TN * (BKIND == CONTIG ? 1 : 2);
-    auto interleave = [&]() {
-#pragma unroll
-        for (int r = 0; r < DS_READS; r++) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-        }
-        if (TM * TN > DS_READS) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - DS_READS, 0);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    // same, with the direct loads of the next step spread between the MFMAs instead of ahead of them
-    auto interleave_loads = [&]() {
-        constexpr int NL = A_LOADS + B_LOADS;
+    auto interleave_loads = [&](int nl) {
         constexpr int NM = TM * TN;
+        constexpr int DS_PER = (DS_READS + NM - 2) / (NM - 1) < 2 ? 2 : (DS_READS + NM - 2) / (NM - 1);
+        int placed = 0, ds_left = DS_READS;
 #pragma unroll
         for (int r = 0; r < NM; r++) {
-            if (r < NL) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);        // 1 VMEM read
-            if (r < DS_READS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                    // 1 MFMA
+            // (the builtin wants literal counts; the conditions fold after unrolling)
+#pragma unroll
+            for (int q = 0; q < DS_PER; q++)
+                if (ds_left > 0) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); ds_left--; }
+            const int want = ((r + 1) * nl + NM - 1) / NM;   // loads due by now
+            if (want - placed >= 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // 1 VMEM read
+            if (want - placed >= 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            if (want - placed >= 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            if (want - placed >= 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            placed = want;
         }
         __builtin_amdgcn_sched_barrier(0);
     };
+    auto interleave = [&]() { interleave_loads(0); };
     // one contraction step on `cur`; `nxt` holds step s+1 when this returns
     auto half_step = [&](char *cur, char *nxt, int s) {
 #pragma unroll
         for (int kk = 0; kk < BK / 16 - 1; kk++) {
+            // the rest of the loads of step s+1 (their stage was released in the previous step)
+            const int lo = LD_T + (kk > 0 ? LD_0 : 0) + (kk > 1 ? LD_1 : 0);
+            const int n = kk == 0 ? LD_0 : (kk == 1 ? LD_1 : LD_2);
+            issue_part(s + 1, nxt, lo, lo + n);
             read_group(cur, kk + 1, (kk + 1) & 1);
             mfma_group(kk & 1);
-            interleave();
+            if (n > 0) interleave_loads(n); else interleave();
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's loads of step s+1 landed
         zero_tail(s + 1, nxt);
         __syncthreads();                     // everyone's did, and nobody reads `cur` any more
-        issue_loads(s + 2, cur);             // past the end on the last steps: harmless re-read
+        issue_part(s + 2, cur, 0, LD_T);
         read_group(nxt, 0, 0);
         mfma_group((BK / 16 - 1) & 1);
-        interleave_loads();
+        if (LD_T > 0) interleave_loads(LD_T); else interleave();
     };
+    // ---- persistent block: walks its share of the logical tiles --------------------------------
+    // Hardware places block b on XCD b % 8.  XCD x owns the contiguous run [x*per, (x+1)*per) of
+    // tiles and its blocks take them round-robin, so the tiles in flight on an XCD at any moment
+    // are neighbours and share operand slices in that XCD's L2; the total % 8 tiles left over go
+    // one each to the blocks of the least loaded slot.
+    const int nbx = gridDim.x / NUM_XCD;
+    const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
+    const int per = p.total_tiles / NUM_XCD, rem = p.total_tiles - per * NUM_XCD;
+    const int n_mine = slot < per ? (per - slot + nbx - 1) / nbx : 0;
+    const int n_all = n_mine + ((xcd < rem && slot == per % nbx) ? 1 : 0);
+    int it = 0;
+    // moves the per-tile state to this block's next tile that has rows; false when there is none
+    auto next_tile = [&]() -> bool {
+        while (it < n_all) {
+            const int logical = it < n_mine ? xcd * per + slot + it * nbx : NUM_XCD * per + xcd;
+            it++;
+            if (setup_tile(logical)) return true;
+        }
+        return false;
+    };
+    bool have = next_tile();
+    bool prefetched = false;   // the loads of step 0 of the current tile are already in flight
+    while (have) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
     // Steps are taken in pairs so the stage names are static; an odd step count (wgrad only: the
     // host requires kc % 128 == 0 otherwise) is padded with a step whose A tile is all zero.
-    const int loop_steps = (total_steps + 1) & ~1;
     if (loop_steps > 0) {
-        issue_loads(0, stage0);
+        if (!prefetched) issue_loads(0, stage0);
         __builtin_amdgcn_s_waitcnt(0x0F70);
         zero_tail(0, stage0);
         __syncthreads();
-        issue_loads(1, stage1);
+        issue_part(1, stage1, 0, LD_T);
         read_group(stage0, 0, 0);
-        for (int step = 0; step < loop_steps; step += 2) {
+        const int n_steps = loop_steps;
+        for (int step = 0; step < n_steps; step += 2) {
             half_step(stage0, stage1, step);
             half_step(stage1, stage0, step + 1);
         }
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the trailing loads before LDS is released
     }
+    __syncthreads();  // the stages are dead: stage 1 becomes the strips, stage 0 the next tile's
+
+    // The next tile's first contraction step is fetched into stage 0 while this tile's results go
+    // out (the strips live in stage 1), which takes the cold-miss latency of a tile's first loads
+    // off the critical path.
+    const int e_expert = expert, e_row_begin = row_begin, e_row_end = row_end, e_n0 = n0;
+    have = next_tile();
+    prefetched = have && loop_steps > 0;
+    if (prefetched) issue_loads(0, stage0);
 
     // ---- epilogue ------------------------------------------------------------------------------
     // Accumulator element r of lane l is output row (l % 32), column (r/4)*8 + (l/32)*4 + (r%4) of
@@ -477,15 +552,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // writes in accumulator layout and the 8-byte reads in row layout are conflict-free) and moves
     // 16 bytes per lane to and from global memory, 64 lanes covering whole 256-byte row segments.
     // The fused SwiGLU backward reads g and u in the same row layout.
-    __syncthreads();  // the stages are dead: reuse them as strips
+    // The epilogue's lane-derived addresses are the same for every tile; recompute them per tile
+    // (a few VALU ops) instead of letting them be hoisted out of the tile loop, where they would
+    // stay live across the main loop and spill.
+    int lane_e = lane, wave_e = __builtin_amdgcn_readfirstlane(wave);
+    asm volatile("" : "+v"(lane_e), "+s"(wave_e));
     constexpr int COLS = (EPI == EPI_SWIGLU) ? WN / 2 : WN;   // output columns of this wavefront
     constexpr int PITCH = COLS * 2 + 8;
     constexpr int STRIP = 32 * PITCH;
     constexpr int NSTRIP = (EPI == EPI_SWIGLU) ? 3 : 1;
     static_assert(NW * NSTRIP * STRIP <= A_BYTES + B_BYTES, "strips must fit in one stage");
-    char *strip = stage0 + wave * (NSTRIP * STRIP);
-    const int lrow = lane & 31;
-    const int lcol = (lane >> 5) * 4;
+    const int wm_e = wave_e / WAVES_N, wn_e = wave_e % WAVES_N;
+    char *strip = stage1 + wave_e * (NSTRIP * STRIP);
+    const int lrow = lane_e & 31;
+    const int lcol = (lane_e >> 5) * 4;
     constexpr int CPRW = COLS / 8;            // 16-byte chunks per strip row
     constexpr int ITS = 32 * CPRW / 64;       // chunks per lane per strip
     // write 4 consecutive columns (as bf16) of row lrow at column `col` of strip `which`
@@ -506,11 +586,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
-    const int col0 = (EPI == EPI_SWIGLU) ? n0 + (wn * WN) / 2 : n0 + wn * WN;   // first output column
-    uint16_t *Cb = p.C + (EPI == EPI_WGRAD ? expert * p.strideC : 0);
+    const int col0 = (EPI == EPI_SWIGLU) ? e_n0 + (wn_e * WN) / 2 : e_n0 + wn_e * WN;   // first output column
+    uint16_t *Cb = p.C + (EPI == EPI_WGRAD ? e_expert * p.strideC : 0);
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-        const int64_t m0 = static_cast<int64_t>(row_begin) + wm * WM + i * 32;  // first row of the strip
+        const int64_t m0 = static_cast<int64_t>(e_row_begin) + wm_e * WM + i * 32;  // first row of the strip
         if (EPI == EPI_SWIGLU) {
 #pragma unroll
             for (int j = 0; j < TN; j += 2)
@@ -540,9 +620,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             u32x4 gq[ITS], uq[ITS];
 #pragma unroll
             for (int it = 0; it < ITS; it++) {
-                const int q = it * 64 + lane;
+                const int q = it * 64 + lane_e;
                 const int64_t m = m0 + q / CPRW;
-                if (m < row_end) {
+                if (m < e_row_end) {
                     const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
                     gq[it] = *reinterpret_cast<const u32x4 *>(p.G + o);
                     uq[it] = *reinterpret_cast<const u32x4 *>(p.U + o);
@@ -550,9 +630,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             }
 #pragma unroll
             for (int it = 0; it < ITS; it++) {
-                const int q = it * 64 + lane;
+                const int q = it * 64 + lane_e;
                 const int64_t m = m0 + q / CPRW;
-                if (m < row_end) {
+                if (m < e_row_end) {
                     float dh[8], gv[8], uv[8], dg[8], du[8];
                     Elem<uint16_t>::unpack(strip_get(0, q / CPRW, q % CPRW), dh);
                     Elem<uint16_t>::unpack(gq[it], gv);
@@ -577,9 +657,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         } else {
 #pragma unroll
             for (int it = 0; it < ITS; it++) {
-                const int q = it * 64 + lane;
+                const int q = it * 64 + lane_e;
                 const int64_t m = m0 + q / CPRW;
-                if (EPI == EPI_WGRAD || m < row_end) {
+                if (EPI == EPI_WGRAD || m < e_row_end) {
                     const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
                     *reinterpret_cast<u32x4 *>(Cb + o) = strip_get(0, q / CPRW, q % CPRW);
                     if (EPI == EPI_SWIGLU) {
@@ -591,6 +671,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         }
         strip_sync();  // the strip is rewritten by the next i
     }
+    __syncthreads();  // the strips alias stage 1, which the next tile loads into
+    }  // tile loop
 }
 
 // ---- host side ---------------------------------------------------------------------------------
@@ -609,6 +691,18 @@ inline bool fits31(int64_t elems) { return elems >= 0 && elems < (1LL << 31); }
 #ifndef OM_WAVES_N
 #define OM_WAVES_N 4
 #endif
+// Blocks of a launch: one resident set (a multiple of the 8 XCDs), or fewer when there are few
+// tiles.  The 256x256 tile's 128 KB of LDS leave room for one block per CU, the 128x128 tile's
+// 64 KB for two.
+constexpr int NUM_CU = 256;
+template <int BM> unsigned persistent_blocks(int64_t tiles) {
+    const int64_t per_xcd_max = (NUM_CU / NUM_XCD) * (BM == 256 ? 1 : 2);
+    int64_t per_xcd = (tiles + NUM_XCD - 1) / NUM_XCD;
+    if (per_xcd > per_xcd_max) per_xcd = per_xcd_max;
+    if (per_xcd < 1) per_xcd = 1;
+    return static_cast<unsigned>(per_xcd * NUM_XCD);
+}
+
 template <int BM> struct Waves {
     static constexpr int M = (BM == 256) ? OM_WAVES_M : 2;
     static constexpr int N = (BM == 256) ? OM_WAVES_N : 2;
@@ -618,10 +712,11 @@ template <int BM, int BN, int AKIND, int BKIND, int EPI>
 int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad family
     constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
     p.m_tiles_max = static_cast<int>((rows + BM - 1) / BM + p.n_experts);
-    const int64_t blocks = static_cast<int64_t>(p.m_tiles_max) * (p.n_cols / BN_OUT);
-    if (blocks > 0x7fffffffLL) return OM_ERR_SHAPE;
+    const int64_t tiles = static_cast<int64_t>(p.m_tiles_max) * (p.n_cols / BN_OUT);
+    if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
+    p.total_tiles = static_cast<int>(tiles);
     ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI>
-        <<<dim3(static_cast<unsigned>(blocks)), dim3(Waves<BM>::M * Waves<BM>::N * 64), 0, st>>>(p);
+        <<<dim3(persistent_blocks<BM>(tiles)), dim3(Waves<BM>::M * Waves<BM>::N * 64), 0, st>>>(p);
     return om_launch_status();
 }
 
@@ -692,12 +787,19 @@ extern "C" int om_grouped_gemm_wgrad(const void *output_grad, const void *input,
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
     hipStream_t st = om_stream(stream);
     if (N % 256 == 0 && K % 256 == 0) {
-        dim3 grid(static_cast<unsigned>((N / 256) * (K / 256)), static_cast<unsigned>(G));
+        p.tiles_e = (N / 256) * (K / 256);
+        const int64_t tiles = static_cast<int64_t>(p.tiles_e) * G;
+        if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
+        p.total_tiles = static_cast<int>(tiles);
         ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD>
-            <<<grid, dim3(Waves<256>::M * Waves<256>::N * 64), 0, st>>>(p);
+            <<<dim3(persistent_blocks<256>(tiles)), dim3(Waves<256>::M * Waves<256>::N * 64), 0, st>>>(p);
     } else {
-        dim3 grid(static_cast<unsigned>((N / 128) * (K / 128)), static_cast<unsigned>(G));
-        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD><<<grid, dim3(256), 0, st>>>(p);
+        p.tiles_e = (N / 128) * (K / 128);
+        const int64_t tiles = static_cast<int64_t>(p.tiles_e) * G;
+        if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
+        p.total_tiles = static_cast<int>(tiles);
+        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD>
+            <<<dim3(persistent_blocks<128>(tiles)), dim3(256), 0, st>>>(p);
     }
     return om_launch_status();
 }
