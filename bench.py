@@ -111,6 +111,32 @@ def bench_moe(args, device):
                 "all_expert_gemms": {"flops_per_step": 9 * prod_flops, "ms_per_step": round(gemm_ms, 3),
                                      "achieved": round(9 * prod_flops / (gemm_ms * 1e-3) / 1e12, 1),
                                      "frac": round(9 * prod_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}}
+    # Yardstick, not part of the metric: the vendor library's dense bf16 GEMM (torch.matmul ->
+    # hipBLASLt) on the two dense shapes with the same row count, contraction and data as the expert
+    # products (one expert's weights for all 131072 rows).  With random operands the chip runs the
+    # matrix cores power-limited, well below its nominal clock, so this is the practical ceiling the
+    # grouped kernels can be held against on the same box.
+    def dense_tflops(a, w):
+        y = torch.empty(a.shape[0], w.shape[0], dtype=a.dtype, device=a.device)
+        for _ in range(3):
+            torch.matmul(a, w.t(), out=y)
+        e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            torch.matmul(a, w.t(), out=y)
+        e1.record(); torch.cuda.synchronize()
+        return 2.0 * a.shape[0] * a.shape[1] * w.shape[0] / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e12
+    with torch.no_grad():
+        a_h = x.detach().reshape(T, H).repeat(K, 1)                       # [TR, H]
+        a_i = torch.randn(TR, I, device=device, dtype=torch.bfloat16)
+        lib_up = dense_tflops(a_h, blk.experts.gate_proj_merged_weight[0])     # [TR,H] x [I,H]^T
+        lib_down = dense_tflops(a_i, blk.experts.down_proj_merged_weight[0])   # [TR,I] x [H,I]^T
+        del a_h, a_i
+    roofline["library_dense_gemm_reference"] = {
+        "what": "torch.matmul bf16 (vendor BLAS) on dense [131072,2048]x[2048,1024] and "
+                "[131072,1024]x[1024,2048], same data distribution, same process",
+        "tflops": [round(lib_up, 1), round(lib_down, 1)],
+        "frac_of_peak": [round(lib_up / PEAK_BF16_TFLOPS, 4), round(lib_down / PEAK_BF16_TFLOPS, 4)]}
     del blk, x, dout
     torch.cuda.empty_cache()
     return dict(T=T, ms_per_step=ms_per_step, roofline=roofline, kernels=kernels, cfg=c)
