@@ -55,6 +55,38 @@ def _require_bf16(*tensors):
 # ----------------------------------------------------------------------------------------------
 # Router
 # ----------------------------------------------------------------------------------------------
+class Fp32LogitsFunction(torch.autograd.Function):
+    """logits = x.float() @ weight.float().T for bf16 x and weight, without the fp32 copies.
+
+    The products of two bf16 values are exact in fp32, so a bf16 GEMM that accumulates and
+    returns fp32 gives what the fp32 GEMM of the up-cast operands gives, up to the order of the
+    sum (reference: modeling_deepseek_v3.py:160 casts both operands to float32 first).  Backward
+    rounds the logits' gradient to bf16 — the precision a bf16 router's backward has anyway — and
+    runs two bf16 GEMMs; the weight gradient is accumulated and returned from fp32."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        ctx.save_for_backward(x, weight)
+        return torch.mm(x, weight.t(), out_dtype=torch.float32)
+
+    @staticmethod
+    def backward(ctx, dlogits):
+        x, weight = ctx.saved_tensors
+        d16 = dlogits.to(torch.bfloat16)
+        dx = torch.mm(d16, weight) if ctx.needs_input_grad[0] else None
+        dw = None
+        if ctx.needs_input_grad[1]:
+            dw = torch.mm(d16.t(), x, out_dtype=torch.float32).to(weight.dtype)
+        return dx, dw
+
+
+def fp32_logits(x, weight):
+    """Router logits in float32 from 2-D x [T,H] and weight [N,H] (the gate's nn.Linear weight)."""
+    if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda:
+        return Fp32LogitsFunction.apply(x.contiguous(), weight.contiguous())
+    return torch.nn.functional.linear(x.float(), weight.float())
+
+
 class SoftmaxTopkRouterFunction(torch.autograd.Function):
     """routing_weights, selected_experts = topk(softmax_fp32(logits), K) [/ sum] -> out dtype.
 
@@ -471,7 +503,7 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
         flat = hidden_states.reshape(-1, hidden_dim)
         if self.router_logits_fp32:
-            router_logits = torch.nn.functional.linear(flat.float(), self.gate.weight.float())
+            router_logits = fp32_logits(flat, self.gate.weight)
         else:
             router_logits = self.gate(flat)
         routing_weights, selected_experts = SoftmaxTopkRouterFunction.apply(

@@ -104,7 +104,7 @@ class DeepseekV3ParallelTopkRouter(nn.Module):
 
     def forward(self, hidden_states):
         hidden_states = hidden_states.reshape(-1, self.config.hidden_size)
-        router_logits = F.linear(hidden_states.type(torch.float32), self.weight.type(torch.float32))
+        router_logits = _moe.fp32_logits(hidden_states, self.weight)
         topk_indices, topk_weights = SigmoidGroupTopkRouterFunction.apply(
             router_logits.contiguous(), self.e_score_correction_bias.float().contiguous(),
             self.n_group, self.topk_group, self.top_k, self.norm_topk_prob,
