@@ -113,6 +113,24 @@ int om_route_softmax_topk_bwd(const void *logits, int logits_dtype, const int64_
                               const void *dweights, int weights_dtype, int64_t T, int N, int K,
                               int norm_topk_prob, void *dlogits, void *stream);
 
+/* om_router_gate_softmax_topk is the whole OLMoE router in one launch: the gate projection
+ *   router_logits = gate(hidden_states) (nn.Linear without bias), optimus/models/common/moe.py:456
+ *   (= optimus/models/olmoe/modeling_olmoe.py:284), followed by :467-471 as above.
+ *   x [T,H] and gate_weight [N,H] are bf16; the logits are accumulated and kept in fp32 (the value
+ *   of x.float() @ gate_weight.float().T up to the order of the sum; a bf16 router rounds them to
+ *   bf16 before the softmax) and written to logits_out [T,N] fp32 when it is not null (the
+ *   backward and output_router_logits need them).  N <= 256, K <= min(N,64), H a multiple of 512
+ *   (256 for N > 64, 64 for N > 128); other shapes return OM_ERR_SHAPE and the caller uses the
+ *   two-step form (library GEMM + om_route_softmax_topk).
+ * om_router_gate_logits is the projection alone, for routers that score the fp32 logits
+ *   differently (optimus/models/deepseek_v3/modeling_deepseek_v3.py:160 casts both operands to
+ *   float32 and calls F.linear).                                                          */
+int om_router_gate_softmax_topk(const void *x, const void *gate_weight, int64_t T, int H, int N,
+                                int K, int norm_topk_prob, float *logits_out, void *weights_out,
+                                int weights_dtype, int64_t *experts_out, void *stream);
+int om_router_gate_logits(const void *x, const void *gate_weight, int64_t T, int H, int N,
+                          float *logits_out, void *stream);
+
 /* om_route_sigmoid_group_topk replaces DeepseekV3ParallelTopkRouter.get_topk_indices and
  *   the weight computation of its forward,
  *   optimus/models/deepseek_v3/modeling_deepseek_v3.py:164-180 and :185-191:

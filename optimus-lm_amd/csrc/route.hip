@@ -256,6 +256,110 @@ __global__ __launch_bounds__(256) void sigmoid_topk_bwd_kernel(const float *__re
     }
 }
 
+// Router gate fused with the routing: logits = x @ Wg^T for 32 tokens per block on the matrix
+// cores (bf16 operands whose products are exact in fp32, fp32 accumulation: the value of
+// x.float() @ Wg.float().T up to the order of the sum), the contraction split over the block's
+// wavefronts and reduced through LDS in a fixed order, then softmax / top-K of those tokens
+// straight from LDS.  x is read from HBM exactly once (the pass is HBM-bound on it); Wg stays in L2.
+// Operand fragments come straight from global memory in MFMA layout (lane = row, 8 consecutive
+// h): the four loads that share a 128-byte line are issued together.
+template <int NB, int WAVES, int UNR, int PER, typename TW, bool ROUTE>
+__global__ __launch_bounds__(WAVES * 64) void gate_route_kernel(
+    const uint16_t *__restrict__ x, const uint16_t *__restrict__ wg, int64_t Tn, int H, int N, int K,
+    int renorm, float *__restrict__ logits_out, TW *__restrict__ weights_out,
+    int64_t *__restrict__ experts_out) {
+    constexpr int NP = NB * 32;  // expert count rounded up to the MFMA block
+    __shared__ float part[WAVES][32][NP];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * 32;
+    const int hw = H / WAVES;
+    const int r32 = lane & 31, kofs = (lane >> 5) * 8;
+    int64_t ta = t0 + r32;
+    if (ta >= Tn) ta = Tn - 1;  // rows past the end: valid memory, result unused
+    const uint16_t *ap = x + ta * H + wave * hw + kofs;
+    const uint16_t *bp[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        int e = j * 32 + r32;
+        if (e >= N) e = N - 1;
+        bp[j] = wg + static_cast<int64_t>(e) * H + wave * hw + kofs;
+    }
+    f32x16 acc[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[j][r] = 0.0f;
+    for (int h = 0; h < hw; h += 16 * UNR) {
+        u32x4 a[UNR], b[NB][UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {
+            a[u] = *reinterpret_cast<const u32x4 *>(ap + h + u * 16);
+#pragma unroll
+            for (int j = 0; j < NB; j++) b[j][u] = *reinterpret_cast<const u32x4 *>(bp[j] + h + u * 16);
+        }
+#pragma unroll
+        for (int u = 0; u < UNR; u++)
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[u]),
+                                                                 __builtin_bit_cast(bf16x8, b[j][u]),
+                                                                 acc[j], 0, 0, 0);
+    }
+    // accumulator element r of lane l: token (r/4)*8 + (l/32)*4 + r%4, expert j*32 + l%32
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            part[wave][(r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)][j * 32 + r32] = acc[j][r];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 32 * NP; idx += WAVES * 64) {
+        const int row = idx / NP, col = idx % NP;
+        float sum = part[0][row][col];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) sum += part[w][row][col];
+        part[0][row][col] = sum;
+        if (logits_out && t0 + row < Tn && col < N) logits_out[(t0 + row) * N + col] = sum;
+    }
+    if (!ROUTE) return;
+    __syncthreads();
+    for (int tk = wave; tk < 32; tk += WAVES) {
+        const int64_t t = t0 + tk;
+        if (t >= Tn) break;
+        float p[PER];
+        row_softmax<PER, float>(&part[0][tk][0], N, lane, p);
+        float w; int e;
+        select_topk<PER>(p, N, K, lane, w, e);
+        if (renorm) {
+            const float sk = wave_sum(lane < K ? w : 0.0f);
+            w = w / sk;
+        }
+        if (lane < K) {
+            Elem<TW>::store(weights_out + t * K + lane, w);
+            experts_out[t * K + lane] = e;
+        }
+    }
+}
+
+template <bool ROUTE, typename TW>
+int launch_gate(const void *x, const void *wg, int64_t T, int H, int N, int K, int renorm,
+                float *logits_out, void *weights_out, int64_t *experts_out, hipStream_t st) {
+    const unsigned nb = static_cast<unsigned>((T + 31) / 32);
+    const uint16_t *xp = static_cast<const uint16_t *>(x), *wp = static_cast<const uint16_t *>(wg);
+    TW *wo = static_cast<TW *>(weights_out);
+#define OM_GATE(NB, WAVES, UNR, PER)                                                              \
+    do {                                                                                          \
+        if (H % (WAVES * 16 * UNR) != 0) return OM_ERR_SHAPE;                                     \
+        gate_route_kernel<NB, WAVES, UNR, PER, TW, ROUTE><<<nb, WAVES * 64, 0, st>>>(             \
+            xp, wp, T, H, N, K, renorm, logits_out, wo, experts_out);                             \
+    } while (0)
+    if (N <= 32) OM_GATE(1, 8, 4, 1);
+    else if (N <= 64) OM_GATE(2, 8, 4, 1);
+    else if (N <= 128) OM_GATE(4, 8, 2, 2);
+    else OM_GATE(8, 4, 1, 4);
+#undef OM_GATE
+    return om_launch_status();
+}
+
 inline unsigned token_blocks(int64_t T) {
     return static_cast<unsigned>((T + TOKENS_PER_BLOCK - 1) / TOKENS_PER_BLOCK);
 }
@@ -349,4 +453,33 @@ extern "C" int om_route_sigmoid_topk_bwd(const float *logits, const int64_t *exp
     OM_DISPATCH_PER(N, (sigmoid_topk_bwd_kernel<PER><<<nb, 256, 0, st>>>(
                            logits, experts, dweights, T, N, K, norm_topk_prob, scale, dlogits)));
     return om_launch_status();
+}
+
+extern "C" int om_router_gate_softmax_topk(const void *x, const void *gate_weight, int64_t T, int H,
+                                           int N, int K, int norm_topk_prob, float *logits_out,
+                                           void *weights_out, int weights_dtype, int64_t *experts_out,
+                                           void *stream) {
+    if (weights_dtype != OM_F32 && weights_dtype != OM_BF16) return OM_ERR_DTYPE;
+    if (T < 0 || H < 1 || H % 8 != 0 || N < 1 || N > 256 || K < 1 || K > N || K > 64 ||
+        T > 0x7fffffffLL)
+        return OM_ERR_SHAPE;
+    if (T == 0) return OM_OK;
+    if (!x || !gate_weight || !weights_out || !experts_out) return OM_ERR_NULL;
+    if (!om_aligned16(x) || !om_aligned16(gate_weight)) return OM_ERR_ALIGN;
+    hipStream_t st = om_stream(stream);
+    if (weights_dtype == OM_F32)
+        return launch_gate<true, float>(x, gate_weight, T, H, N, K, norm_topk_prob, logits_out,
+                                        weights_out, experts_out, st);
+    return launch_gate<true, uint16_t>(x, gate_weight, T, H, N, K, norm_topk_prob, logits_out,
+                                       weights_out, experts_out, st);
+}
+
+extern "C" int om_router_gate_logits(const void *x, const void *gate_weight, int64_t T, int H, int N,
+                                     float *logits_out, void *stream) {
+    if (T < 0 || H < 1 || H % 8 != 0 || N < 1 || N > 256 || T > 0x7fffffffLL) return OM_ERR_SHAPE;
+    if (T == 0) return OM_OK;
+    if (!x || !gate_weight || !logits_out) return OM_ERR_NULL;
+    if (!om_aligned16(x) || !om_aligned16(gate_weight)) return OM_ERR_ALIGN;
+    return launch_gate<false, float>(x, gate_weight, T, H, N, 1, 0, logits_out, nullptr, nullptr,
+                                     om_stream(stream));
 }

@@ -37,6 +37,9 @@ SIGNATURES = {
                                       c_void_p, c_void_p]),
     "om_route_softmax_topk_bwd": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_i64, c_int,
                                           c_int, c_int, c_void_p, c_void_p]),
+    "om_router_gate_softmax_topk": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_int, c_int,
+                                            c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
+    "om_router_gate_logits": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p, c_void_p]),
     "om_route_sigmoid_group_topk": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_int, c_int,
                                             c_int, c_double, c_void_p, c_void_p, c_void_p]),
     "om_route_sigmoid_topk_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int, c_int,

@@ -80,11 +80,89 @@ class Fp32LogitsFunction(torch.autograd.Function):
         return dx, dw
 
 
+def gate_kernel_fits(x, weight):
+    """Shapes and dtypes the fused gate kernels take (om_router_gate_*)."""
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
+        return False
+    N, H = weight.shape
+    if N > 256 or x.shape[0] == 0:
+        return False
+    return H % (512 if N <= 64 else 256 if N <= 128 else 64) == 0
+
+
+def _gate_backward(x, weight, dlogits, needs):
+    """(dx, dweight) of logits = x @ weight.T from the fp32 gradient of the logits: rounded to bf16
+    (the precision a bf16 router's backward has anyway), two library GEMMs, the weight gradient
+    accumulated in fp32."""
+    d16 = dlogits.to(torch.bfloat16)
+    dx = torch.mm(d16, weight) if needs[0] else None
+    dw = torch.mm(d16.t(), x, out_dtype=torch.float32).to(weight.dtype) if needs[1] else None
+    return dx, dw
+
+
+class GateLogitsFunction(torch.autograd.Function):
+    """fp32 logits of a bf16 gate through om_router_gate_logits (one pass over x)."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        T, (N, H) = x.shape[0], weight.shape
+        logits = torch.empty((T, N), dtype=torch.float32, device=x.device)
+        _n.check(_n.lib().om_router_gate_logits(_n.ptr(x), _n.ptr(weight), T, H, N, _n.ptr(logits),
+                                                _n.stream()), "om_router_gate_logits")
+        ctx.save_for_backward(x, weight)
+        return logits
+
+    @staticmethod
+    def backward(ctx, dlogits):
+        x, weight = ctx.saved_tensors
+        return _gate_backward(x, weight, dlogits, ctx.needs_input_grad)
+
+
 def fp32_logits(x, weight):
     """Router logits in float32 from 2-D x [T,H] and weight [N,H] (the gate's nn.Linear weight)."""
+    if gate_kernel_fits(x, weight):
+        return GateLogitsFunction.apply(x.contiguous(), weight.contiguous())
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda:
         return Fp32LogitsFunction.apply(x.contiguous(), weight.contiguous())
     return torch.nn.functional.linear(x.float(), weight.float())
+
+
+class GateSoftmaxTopkFunction(torch.autograd.Function):
+    """The OLMoE router in one launch (om_router_gate_softmax_topk): gate projection with fp32
+    logits, softmax, top-K, optional renormalisation.  Returns (routing_weights, selected_experts,
+    router_logits fp32); reference moe.py:456 and :467-471."""
+
+    @staticmethod
+    def forward(ctx, x, weight, top_k, norm_topk_prob, out_dtype):
+        T, (N, H) = x.shape[0], weight.shape
+        dev = x.device
+        logits = torch.empty((T, N), dtype=torch.float32, device=dev)
+        weights = torch.empty((T, top_k), dtype=out_dtype, device=dev)
+        experts = torch.empty((T, top_k), dtype=torch.int64, device=dev)
+        _n.check(_n.lib().om_router_gate_softmax_topk(
+            _n.ptr(x), _n.ptr(weight), T, H, N, top_k, int(bool(norm_topk_prob)), _n.ptr(logits),
+            _n.ptr(weights), _n.dtype_code(weights), _n.ptr(experts), _n.stream()),
+            "om_router_gate_softmax_topk")
+        ctx.save_for_backward(x, weight, logits, experts)
+        ctx.norm_topk_prob = bool(norm_topk_prob)
+        ctx.mark_non_differentiable(experts)
+        return weights, experts, logits
+
+    @staticmethod
+    def backward(ctx, weights_grad, _experts_grad, logits_grad):
+        x, weight, logits, experts = ctx.saved_tensors
+        T, N = logits.shape
+        K = experts.shape[1]
+        weights_grad = weights_grad.contiguous()
+        dlogits = torch.empty_like(logits)
+        _n.check(_n.lib().om_route_softmax_topk_bwd(
+            _n.ptr(logits), _n.OM_F32, _n.ptr(experts), _n.ptr(weights_grad),
+            _n.dtype_code(weights_grad), T, N, K, int(ctx.norm_topk_prob), _n.ptr(dlogits),
+            _n.stream()), "om_route_softmax_topk_bwd")
+        if logits_grad is not None:
+            dlogits = dlogits + logits_grad
+        dx, dw = _gate_backward(x, weight, dlogits, ctx.needs_input_grad)
+        return dx, dw, None, None, None
 
 
 class SoftmaxTopkRouterFunction(torch.autograd.Function):
@@ -502,13 +580,18 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
     def forward(self, hidden_states):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
         flat = hidden_states.reshape(-1, hidden_dim)
-        if self.router_logits_fp32:
-            router_logits = fp32_logits(flat, self.gate.weight)
+        if self.router_logits_fp32 and gate_kernel_fits(flat, self.gate.weight):
+            routing_weights, selected_experts, router_logits = GateSoftmaxTopkFunction.apply(
+                flat.contiguous(), self.gate.weight, self.num_experts_per_tok, self.norm_topk_prob,
+                hidden_states.dtype)
         else:
-            router_logits = self.gate(flat)
-        routing_weights, selected_experts = SoftmaxTopkRouterFunction.apply(
-            router_logits.contiguous(), self.num_experts_per_tok, self.norm_topk_prob,
-            hidden_states.dtype)
+            if self.router_logits_fp32:
+                router_logits = fp32_logits(flat, self.gate.weight)
+            else:
+                router_logits = self.gate(flat)
+            routing_weights, selected_experts = SoftmaxTopkRouterFunction.apply(
+                router_logits.contiguous(), self.num_experts_per_tok, self.norm_topk_prob,
+                hidden_states.dtype)
 
         def expert_computation_block(hidden_states, selected_experts, routing_weights):
             b, s, h = hidden_states.shape

@@ -133,3 +133,78 @@ def test_sigmoid_group_topk(cuda, T, N, n_group, topk_group, K, renorm):
         wr = wr / (wr.sum(-1, keepdim=True) + 1e-20)
     (wr * 2.5).backward(dw)
     assert float((x.grad.cpu() - lr.grad).abs().max()) <= 1e-5 * max(1.0, float(lr.grad.abs().max()))
+
+
+# ---- gate projection fused with the routing (om_router_gate_logits / om_router_gate_softmax_topk) --
+def _gate_inputs(T, H, N, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, H, generator=g) * 0.02).to(torch.bfloat16)
+    return x, w
+
+
+@pytest.mark.parametrize("T,H,N", [(1000, 2048, 64), (64, 512, 8), (33, 1024, 128), (300, 7168, 256),
+                                   (4096, 2048, 60)])
+def test_gate_logits_match_fp32_matmul(cuda, T, H, N):
+    """fp32 logits from bf16 operands: the products are exact, only the order of the fp32 sum differs
+    from the CPU matmul of the up-cast operands."""
+    from optimus.models.common.moe import fp32_logits, gate_kernel_fits
+    x, w = _gate_inputs(T, H, N, seed=T + N)
+    assert gate_kernel_fits(x.to(cuda), w.to(cuda))
+    got = fp32_logits(x.to(cuda), w.to(cuda)).cpu()
+    ref = x.float() @ w.float().t()
+    exact = (x.double() @ w.double().t())
+    assert got.dtype == torch.float32 and got.shape == (T, N)
+    # both are fp32 sums of the same exact products: compare their distance to the fp64 value
+    err_got = float((got.double() - exact).abs().max()); err_ref = float((ref.double() - exact).abs().max())
+    assert err_got <= max(4 * err_ref, 2e-6), (err_got, err_ref)
+
+
+@pytest.mark.parametrize("T,H,N,K,renorm,wdt", [
+    (16384, 2048, 64, 8, False, torch.bfloat16),    # C3
+    (1000, 2048, 64, 8, True, torch.float32),       # ragged token count
+    (512, 1024, 128, 6, True, torch.float32),
+    (96, 512, 8, 2, True, torch.bfloat16),
+])
+def test_gate_softmax_topk_equals_two_step_on_its_own_logits(cuda, T, H, N, K, renorm, wdt):
+    """The routing half of the fused kernel is the same code as om_route_softmax_topk: on the logits
+    the kernel itself returns, experts and weights must be identical bit for bit, and the experts
+    equal the CPU oracle's on rows without near-ties."""
+    from optimus.models.common.moe import GateSoftmaxTopkFunction, SoftmaxTopkRouterFunction
+    x, w = _gate_inputs(T, H, N, seed=7 * T + N)
+    wts, exp, logits = GateSoftmaxTopkFunction.apply(x.to(cuda), w.to(cuda), K, renorm, wdt)
+    w2, e2 = SoftmaxTopkRouterFunction.apply(logits.contiguous(), K, renorm, wdt)
+    assert torch.equal(exp, e2) and torch.equal(wts.view(torch.int16 if wdt == torch.bfloat16 else torch.int32),
+                                                w2.view(torch.int16 if wdt == torch.bfloat16 else torch.int32))
+    lg = logits.cpu()
+    w_ref, e_ref, _ = R.olmoe_router(lg, K, renorm, wdt)
+    probs = torch.softmax(lg, 1)
+    top = torch.sort(probs, dim=1, descending=True).values[:, :K + 1]
+    ok = ((top[:, :-1] - top[:, 1:]) > 4 * top[:, :-1] * 2.0 ** -23).all(dim=1)
+    assert int(ok.sum()) >= 0.99 * T and torch.equal(exp.cpu()[ok], e_ref[ok])
+
+
+def test_gate_softmax_topk_backward(cuda):
+    """dx and dW of the fused router against autograd of the fp32 restatement (the gradient of the
+    logits is rounded to bf16 before the two GEMMs, as a bf16 router's backward does)."""
+    from optimus.models.common.moe import GateSoftmaxTopkFunction
+    T, H, N, K = 2048, 1024, 64, 8
+    x, w = _gate_inputs(T, H, N, seed=5)
+    g = torch.Generator().manual_seed(6)
+    dw_out = torch.randn(T, K, generator=g)
+    dlogit_out = torch.randn(T, N, generator=g) * 0.1
+    xg = x.to(cuda).requires_grad_(True); wg = w.to(cuda).requires_grad_(True)
+    wts, exp, logits = GateSoftmaxTopkFunction.apply(xg, wg, K, True, torch.float32)
+    (wts * dw_out.to(cuda)).sum().backward(retain_graph=True)
+    gx1, gw1 = xg.grad.clone(), wg.grad.clone()
+    xg.grad = None; wg.grad = None
+    ((wts * dw_out.to(cuda)).sum() + (logits * dlogit_out.to(cuda)).sum()).backward()
+    # reference in fp32 on the CPU with the kernel's own expert choice
+    xr = x.float().requires_grad_(True); wr = w.float().requires_grad_(True)
+    lr = xr @ wr.t()
+    pr = torch.softmax(lr, 1).gather(1, exp.cpu())
+    pr = pr / pr.sum(1, keepdim=True)
+    ((pr * dw_out).sum() + (lr * dlogit_out).sum()).backward()
+    rel = lambda a, b: float((a.float().cpu() - b).abs().mean() / b.abs().mean())
+    assert rel(xg.grad, xr.grad) < 1e-2 and rel(wg.grad, wr.grad) < 1e-2
+    assert not torch.equal(gx1, xg.grad)     # the logits' own gradient takes part
