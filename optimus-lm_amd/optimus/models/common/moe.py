@@ -622,3 +622,55 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
                     self.experts.down_proj_merged_weight[local_expert_idx].copy_(src.down_proj.weight.data)
                 else:
                     self.experts[local_expert_idx].load_state_dict(src.state_dict())
+
+
+# ----------------------------------------------------------------------------------------------
+# Checkpoint interchange between the merged and the per-expert weight layouts
+# ----------------------------------------------------------------------------------------------
+_MERGED_SUFFIX = "_merged_weight"
+
+
+def merged_state_dict_to_per_expert(state_dict, expert_start_id=0):
+    """Rewrites '<p>.experts.<lin>_merged_weight' [NR,out,in] entries as NR entries
+    '<p>.experts.<id>.<lin>.weight' (views, no copies), id = expert_start_id + local index; all
+    other entries pass through.  This is the un-merging the reference does when it converts an
+    expert-parallel rank's checkpoint to per-expert keys
+    (evals/convert_olmoe_om_checkpoint_to_hf.py:59-88)."""
+    out = {}
+    for name, tensor in state_dict.items():
+        tokens = name.split(".")
+        if "experts" in tokens and tokens[-1].endswith(_MERGED_SUFFIX):
+            linear_key = tokens[-1][: -len(_MERGED_SUFFIX)]
+            for local in range(tensor.shape[0]):
+                serial = ".".join(tokens[:-1] + [str(expert_start_id + local), linear_key, "weight"])
+                out[serial] = tensor[local]
+        else:
+            out[name] = tensor
+    return out
+
+
+def per_expert_state_dict_to_merged(state_dict, num_local_experts, expert_start_id=0):
+    """The inverse: gathers '<p>.experts.<id>.<lin>.weight' for id in
+    [expert_start_id, expert_start_id + num_local_experts) into '<p>.experts.<lin>_merged_weight'
+    (one stacked tensor per projection); entries of experts outside the window are dropped, all
+    other entries pass through.  Same mapping as the reference's checkpoint generator for
+    use_merged_mlp_in_fast_moe (generate_parallel_model.py:136-148)."""
+    out, groups = {}, {}
+    for name, tensor in state_dict.items():
+        tokens = name.split(".")
+        if "experts" in tokens:
+            i = tokens.index("experts")
+            if len(tokens) == i + 4 and tokens[i + 1].isdigit() and tokens[-1] == "weight":
+                local = int(tokens[i + 1]) - expert_start_id
+                if 0 <= local < num_local_experts:
+                    key = ".".join(tokens[: i + 1] + [tokens[i + 2] + _MERGED_SUFFIX])
+                    groups.setdefault(key, {})[local] = tensor
+                continue
+        out[name] = tensor
+    for key, parts in groups.items():
+        missing = [expert_start_id + j for j in range(num_local_experts) if j not in parts]
+        if missing:
+            raise KeyError(f"{key}: no weights for experts {missing}")
+        out[key] = torch.stack([parts[j] for j in range(num_local_experts)])
+    return out
+

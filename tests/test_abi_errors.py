@@ -1,0 +1,99 @@
+"""Error convention of the C ABI: every entry point validates its arguments before it touches the
+HIP runtime and answers with a negative OM_ERR_* code — it never throws and never launches on bad
+input.  These calls return from the validation, so they run without a GPU; the pointers are made-up
+addresses that are never dereferenced on the host."""
+import pytest
+
+from optimus import _native as n
+
+OK, NULL, DTYPE, SHAPE, ALIGN, LAUNCH, WORKSPACE = 0, -1, -2, -3, -4, -5, -6
+P = 0x7f0000001000        # a 16-byte aligned, never dereferenced "device pointer"
+ODD = P + 8               # misaligned
+BF16, F32, I64 = n.OM_BF16, n.OM_F32, 1
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return n.lib()
+
+
+def test_strerror_names_every_code(lib):
+    texts = {c: lib.om_strerror(c).decode() for c in (OK, NULL, DTYPE, SHAPE, ALIGN, LAUNCH, WORKSPACE)}
+    assert len(set(texts.values())) == 7 and all(texts.values())
+    assert "unknown" in lib.om_strerror(-99).decode()
+
+
+def test_adamw(lib):
+    hp = (4e-4, 0.9, 0.95, 1e-8, 0.1)
+    assert lib.om_adamw_step(P, P, P, P, P, 16, *hp, 1, 7, None) == DTYPE
+    assert lib.om_adamw_step(P, P, P, P, P, 16, *hp, 0, BF16, None) == SHAPE      # step is 1-based
+    assert lib.om_adamw_step(P, P, P, P, P, -1, *hp, 1, BF16, None) == SHAPE
+    assert lib.om_adamw_step(P, P, P, P, P, 0, *hp, 1, BF16, None) == OK          # nothing to do
+    assert lib.om_adamw_step(P, None, P, P, P, 16, *hp, 1, BF16, None) == NULL
+    assert lib.om_adamw_step(None, P, P, P, P, 16, *hp, 1, BF16, None) == NULL    # bf16 mode needs param
+    assert lib.om_adamw_step(P, P, ODD, P, P, 16, *hp, 1, BF16, None) == ALIGN
+    assert lib.om_adamw_step_clipped(P, P, P, P, P, 16, *hp, 1, BF16, None, 1, None) == NULL   # no scale
+    assert lib.om_adamw_step_clipped(P, P, P, P, P, 16, *hp, 1, 9, P, 1, None) == DTYPE
+
+
+def test_grad_norm(lib):
+    assert lib.om_grad_sumsq(P, 5, P, 4, P, None) == DTYPE
+    assert lib.om_grad_sumsq(P, BF16, P, -1, P, None) == SHAPE
+    assert lib.om_grad_sumsq(P, BF16, P, 0, P, None) == OK
+    assert lib.om_grad_sumsq(None, BF16, P, 4, P, None) == NULL
+    assert lib.om_grad_sumsq(ODD, BF16, P, 4, P, None) == ALIGN
+    assert lib.om_grad_norm_clip_coef(P, P, 0, BF16, 1.0, P, P, P, None) == SHAPE
+    assert lib.om_grad_norm_clip_coef(P, P, 3, BF16, 1.0, None, P, P, None) == NULL
+    assert lib.om_grad_norm_clip_coef(P, P, 3, 4, 1.0, P, P, P, None) == DTYPE
+
+
+def test_routers(lib):
+    assert lib.om_route_softmax_topk(P, 3, 8, 64, 8, 0, P, BF16, P, None) == DTYPE
+    assert lib.om_route_softmax_topk(P, F32, 8, 600, 8, 0, P, BF16, P, None) == SHAPE      # N > 512
+    assert lib.om_route_softmax_topk(P, F32, 8, 4, 8, 0, P, BF16, P, None) == SHAPE        # K > N
+    assert lib.om_route_softmax_topk(P, F32, 0, 64, 8, 0, P, BF16, P, None) == OK
+    assert lib.om_route_softmax_topk(None, F32, 8, 64, 8, 0, P, BF16, P, None) == NULL
+    assert lib.om_route_softmax_topk_bwd(P, F32, None, P, BF16, 8, 64, 8, 0, P, None) == NULL
+    assert lib.om_route_sigmoid_group_topk(P, P, 8, 256, 7, 4, 8, 1, 2.5, P, P, None) == SHAPE   # 256 % 7
+    assert lib.om_route_sigmoid_group_topk(P, None, 8, 256, 8, 4, 8, 1, 2.5, P, P, None) == NULL
+    assert lib.om_router_gate_softmax_topk(P, P, 8, 2048, 300, 8, 0, P, P, BF16, P, None) == SHAPE   # N > 256
+    assert lib.om_router_gate_softmax_topk(P, P, 8, 2000, 64, 8, 0, P, P, BF16, P, None) == SHAPE   # H % 512
+    assert lib.om_router_gate_softmax_topk(ODD, P, 8, 2048, 64, 8, 0, P, P, BF16, P, None) == ALIGN
+    assert lib.om_router_gate_softmax_topk(P, P, 8, 2048, 64, 8, 0, P, None, BF16, P, None) == NULL
+    assert lib.om_router_gate_logits(P, P, 8, 2048, 64, None, None) == NULL
+
+
+def test_sort_and_index_ops(lib):
+    need = lib.om_moe_sort_workspace_bytes(1024, 8, 64)
+    assert need > 0
+    assert lib.om_moe_sort(P, 5, 1024, 8, 0, 64, P, P, P, P, P, P, need, None) == DTYPE
+    assert lib.om_moe_sort(P, I64, 1024, 0, 0, 64, P, P, P, P, P, P, need, None) == SHAPE
+    assert lib.om_moe_sort(P, I64, 1024, 8, 0, 64, None, P, P, P, P, P, need, None) == NULL
+    assert lib.om_moe_sort(P, I64, 1024, 8, 0, 64, P, P, P, P, P, P, need - 1, None) == WORKSPACE
+    assert lib.om_compute_partial_token_counts(P, I64, P, P, 0, 64, 1000, 8, 64, None) == SHAPE   # T % TH
+    assert lib.om_index_gather(P, P, P, 16, 64, 3, None) == DTYPE
+    assert lib.om_index_gather(P, None, P, 16, 64, BF16, None) == NULL
+    assert lib.om_index_gather(P, P, P, 0, 64, BF16, None) == OK
+    assert lib.om_index_add(P, P, P, -1, 64, BF16, None) == SHAPE
+    assert lib.om_swiglu_fwd(P, P, ODD, 64, BF16, None) == ALIGN
+    assert lib.om_swiglu_bwd(P, P, P, None, P, 64, BF16, None) == NULL
+
+
+def test_grouped_gemms(lib):
+    args = (131072, 64, 2048, 1024, 0, None)
+    assert lib.om_grouped_gemm_fwd(P, P, P, P, 131072, 64, 2000, 1024, 0, None) == SHAPE    # N % 128
+    assert lib.om_grouped_gemm_fwd(P, P, P, P, 0, 64, 2048, 1024, 0, None) == OK            # no rows
+    assert lib.om_grouped_gemm_fwd(P, None, P, P, *args) == NULL
+    assert lib.om_grouped_gemm_fwd(P, P, ODD, P, *args) == ALIGN
+    assert lib.om_grouped_gemm_fwd(P, P, P, P, 1 << 22, 64, 2048, 1024, 0, None) == SHAPE   # > 2^31 elements
+    assert lib.om_grouped_gemm_dgrad(P, P, P, None, *args) == NULL
+    assert lib.om_grouped_gemm_wgrad(P, P, P, P, 131072, 0, 2048, 1024, 0, None) == SHAPE   # G < 1
+    assert lib.om_merged_mlp_gate_up_fwd(P, P, P, P, P, P, P, 131072, 64, 1000, 2048, 0, None) == SHAPE
+    assert lib.om_merged_mlp_gate_up_fwd(P, P, None, P, P, P, P, 131072, 64, 1024, 2048, 0, None) == NULL
+    assert lib.om_merged_mlp_down_dgrad(P, P, P, P, P, ODD, P, 131072, 64, 1024, 2048, 0, None) == ALIGN
+    assert lib.om_merged_mlp_gate_up_dgrad(P, P, P, P, None, P, 131072, 64, 1024, 2048, 0, None) == NULL
+
+
+def test_check_raises_with_the_library_text():
+    with pytest.raises(n.NativeLibraryError, match="dtype"):
+        n.check(DTYPE, "om_adamw_step")
