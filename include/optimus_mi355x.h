@@ -131,6 +131,24 @@ int om_router_gate_softmax_topk(const void *x, const void *gate_weight, int64_t 
 int om_router_gate_logits(const void *x, const void *gate_weight, int64_t T, int H, int N,
                           float *logits_out, void *stream);
 
+/* Load-balancing statistics of one layer's router logits
+ * replaces: the per-token part of load_balancing_loss_func,
+ *   optimus/models/olmoe/modeling_olmoe.py:44-57 (softmax, top-K, one-hot mean, probability
+ *   mean), and of single_input_/layer_level_load_balancing_loss_func,
+ *   optimus/models/common/ral_functions.py:6-35.
+ * prob_sum[e] = sum over tokens of softmax(logits[t,:])[e] (fp32);
+ * count[e]    = number of tokens whose top-K (probability desc, expert index asc) holds e, as float.
+ * The loss is num_experts * sum_e (count[e]/T) * (prob_sum[e]/T); the means and the product are
+ * left to the caller, who may combine several layers.  workspace: om_router_balance_workspace_bytes.
+ * om_router_balance_bwd: dlogits[t,i] = p_i * (g_i - sum_j p_j g_j) with g = prob_grad [N] fp32,
+ *   the gradient of the loss with respect to prob_sum (the counts carry no gradient).      */
+int64_t om_router_balance_workspace_bytes(int64_t T, int N);
+int om_router_balance_stats(const void *logits, int logits_dtype, int64_t T, int N, int K,
+                            float *prob_sum, float *count, void *workspace,
+                            int64_t workspace_bytes, void *stream);
+int om_router_balance_bwd(const void *logits, int logits_dtype, const float *prob_grad, int64_t T,
+                          int N, void *dlogits, void *stream);
+
 /* om_route_sigmoid_group_topk replaces DeepseekV3ParallelTopkRouter.get_topk_indices and
  *   the weight computation of its forward,
  *   optimus/models/deepseek_v3/modeling_deepseek_v3.py:164-180 and :185-191:

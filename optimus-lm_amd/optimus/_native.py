@@ -40,6 +40,10 @@ SIGNATURES = {
     "om_router_gate_softmax_topk": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_int, c_int,
                                             c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
     "om_router_gate_logits": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p, c_void_p]),
+    "om_router_balance_workspace_bytes": (c_i64, [c_i64, c_int]),
+    "om_router_balance_stats": (c_int, [c_void_p, c_int, c_i64, c_int, c_int, c_void_p, c_void_p,
+                                        c_void_p, c_i64, c_void_p]),
+    "om_router_balance_bwd": (c_int, [c_void_p, c_int, c_void_p, c_i64, c_int, c_void_p, c_void_p]),
     "om_route_sigmoid_group_topk": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_int, c_int,
                                             c_int, c_double, c_void_p, c_void_p, c_void_p]),
     "om_route_sigmoid_topk_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int, c_int,
@@ -84,7 +88,8 @@ _lib = None
 # appends (name, start_event, end_event) recorded on the current stream.  Used by bench.py to get
 # kernel durations from HIP events inside the timed region; None (the default) costs one test.
 launch_log = None
-_UNTIMED = {"om_version", "om_arch", "om_strerror", "om_moe_sort_workspace_bytes"}
+_UNTIMED = {"om_version", "om_arch", "om_strerror", "om_moe_sort_workspace_bytes",
+            "om_router_balance_workspace_bytes"}
 
 
 class NativeLibraryError(RuntimeError):

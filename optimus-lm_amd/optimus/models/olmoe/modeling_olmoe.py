@@ -14,6 +14,8 @@ import torch.nn as nn
 from torch.utils.checkpoint import checkpoint as torch_activation_checkpoint
 
 from optimus.models.common import moe as _moe
+from optimus.models.common.ral_functions import (  # noqa: F401  (same names as the reference module)
+    layer_level_load_balancing_loss_func, load_balancing_loss_func)
 
 
 class OlmoeParallelMLP(nn.Module):

@@ -71,3 +71,27 @@ def dsv3_router(hidden_states, weight, bias, n_group, topk_group, top_k, norm_to
         topk_weights = topk_weights / denominator
     topk_weights = topk_weights * routed_scaling_factor                               # :191
     return topk_indices, topk_weights, router_logits
+
+
+def load_balancing_loss(gate_logits, num_experts, top_k):
+    """The reference's global auxiliary loss without a mask, optimus/models/olmoe/modeling_olmoe.py:
+    39-46 and :84-85, as the torch expressions it uses (softmax, topk, one_hot, two means), in the
+    dtype of the logits.  `gate_logits` is a tuple of per-layer [T,N] tensors."""
+    cat = torch.cat(list(gate_logits), dim=0)                                        # :41
+    routing_weights = torch.nn.functional.softmax(cat, dim=-1)                       # :43
+    _, selected = torch.topk(routing_weights, top_k, dim=-1)                         # :45
+    expert_mask = torch.nn.functional.one_hot(selected, num_experts)                 # :47
+    tokens_per_expert = torch.mean(expert_mask.float(), dim=0)                       # :51
+    router_prob_per_expert = torch.mean(routing_weights, dim=0)                      # :54
+    return torch.sum(tokens_per_expert * router_prob_per_expert.unsqueeze(0)) * num_experts   # :84-85
+
+
+def layer_level_load_balancing_loss(gate_logits, num_experts, top_k):
+    """optimus/models/common/ral_functions.py:18-35: the same per layer, summed over the layers."""
+    stacked = torch.stack(list(gate_logits), dim=0)
+    routing_weights = torch.nn.functional.softmax(stacked, dim=-1)
+    _, selected = torch.topk(routing_weights, top_k, dim=-1)
+    expert_mask = torch.nn.functional.one_hot(selected, num_experts)
+    tokens_per_expert = torch.mean(expert_mask.float(), dim=1)
+    router_prob_per_expert = torch.mean(routing_weights, dim=1)
+    return torch.sum(tokens_per_expert * router_prob_per_expert.unsqueeze(1)) * num_experts

@@ -208,3 +208,39 @@ def test_gate_softmax_topk_backward(cuda):
     rel = lambda a, b: float((a.float().cpu() - b).abs().mean() / b.abs().mean())
     assert rel(xg.grad, xr.grad) < 1e-2 and rel(wg.grad, wr.grad) < 1e-2
     assert not torch.equal(gx1, xg.grad)     # the logits' own gradient takes part
+
+
+# ---- auxiliary load-balancing loss (om_router_balance_stats / _bwd) ---------------------------------
+@pytest.mark.parametrize("L,T,N,K", [(3, 4096, 64, 8), (2, 1000, 100, 5), (1, 77, 256, 8), (4, 512, 8, 2)])
+def test_balance_losses_match_the_reference_expressions(cuda, L, T, N, K):
+    from optimus.models.common.ral_functions import (layer_level_load_balancing_loss_func,
+                                                     load_balancing_loss_func,
+                                                     single_input_load_balancing_loss_func)
+    layers = tuple(_valid_logits(T, N, K, seed=31 * l + T) for l in range(L))
+    dev = tuple(l.to(cuda) for l in layers)
+    got = float(load_balancing_loss_func(dev, N, K)); want = float(R.load_balancing_loss(layers, N, K))
+    assert abs(got - want) <= 2e-5 * want
+    got = float(layer_level_load_balancing_loss_func(dev, N, K))
+    want = float(R.layer_level_load_balancing_loss(layers, N, K))
+    assert abs(got - want) <= 2e-5 * want
+    got = float(single_input_load_balancing_loss_func(dev[0], N, K))
+    want = float(R.load_balancing_loss(layers[:1], N, K))
+    assert abs(got - want) <= 2e-5 * want
+    assert load_balancing_loss_func(None, N, K) == 0 and load_balancing_loss_func(dev[0], N, K) == 0
+
+
+def test_balance_loss_gradient_and_bf16_logits(cuda):
+    from optimus.models.common.ral_functions import load_balancing_loss_func
+    L, T, N, K = 2, 2048, 64, 8
+    layers = [_valid_logits(T, N, K, seed=77 + l) for l in range(L)]
+    ref = [l.clone().requires_grad_(True) for l in layers]
+    R.load_balancing_loss(tuple(ref), N, K).backward()
+    dev = [l.to(cuda).requires_grad_(True) for l in layers]
+    load_balancing_loss_func(tuple(dev), N, K).backward()
+    for a, b in zip(dev, ref):
+        assert float((a.grad.cpu() - b.grad).abs().max()) <= 1e-5 * float(b.grad.abs().max())
+    # bf16 logits: probabilities are kept in fp32 here, rounded to bf16 in the reference
+    b16 = tuple(l.to(torch.bfloat16) for l in layers)
+    got = float(load_balancing_loss_func(tuple(l.to(cuda) for l in b16), N, K))
+    want = float(R.load_balancing_loss(tuple(l.float() for l in b16), N, K))
+    assert abs(got - want) <= 1e-3 * want

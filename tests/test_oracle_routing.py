@@ -1,6 +1,7 @@
 """Pins the router restatements (oracle/routing.py) against the library calls the reference makes
 (torch.softmax, torch.topk) on tie-free rows, their invariants, and a brute-force statement of the
 DeepSeek-V3 group-limited selection on a tiny shape."""
+import math
 import itertools
 
 import pytest
@@ -84,3 +85,47 @@ def test_dsv3_router_invariants_and_library_topk():
     score_mask = mask.unsqueeze(-1).expand(-1, 8, 32).reshape(T, N)
     ref = torch.topk(sfc.masked_fill(~score_mask.bool(), 0.0), k=8, dim=-1, sorted=False)[1]
     assert torch.equal(torch.sort(e, 1).values, torch.sort(ref, 1).values)
+
+
+# ---- auxiliary load-balancing loss ------------------------------------------------------------
+def _brute_force_balance_loss(logits, N, K):
+    """Token-by-token statement: c[e] = share of tokens with e among their K most probable experts,
+    P[e] = mean probability; loss = N * sum_e c[e] P[e]."""
+    T = logits.shape[0]
+    c = [0.0] * N; P = [0.0] * N
+    for t in range(T):
+        row = [float(v) for v in logits[t].double()]
+        m = max(row); ex = [math.exp(v - m) for v in row]; z = sum(ex)
+        p = [v / z for v in ex]
+        order = sorted(range(N), key=lambda i: (-p[i], i))[:K]
+        for e in order:
+            c[e] += 1.0 / T
+        for e in range(N):
+            P[e] += p[e] / T
+    return N * sum(ci * pi for ci, pi in zip(c, P))
+
+
+def test_balance_loss_restatement_vs_brute_force():
+    g = torch.Generator().manual_seed(3)
+    layers = tuple(torch.randn(40, 12, generator=g) for _ in range(3))
+    want = _brute_force_balance_loss(torch.cat(layers), 12, 3)
+    got = float(R.load_balancing_loss(layers, 12, 3))
+    assert abs(got - want) <= 1e-5 * want
+    per_layer = sum(_brute_force_balance_loss(l, 12, 3) for l in layers)
+    assert abs(float(R.layer_level_load_balancing_loss(layers, 12, 3)) - per_layer) <= 1e-5 * per_layer
+
+
+def test_balance_loss_closed_forms():
+    # every token has the same logits: the K most probable experts get all the tokens
+    row = torch.tensor([0.3, 2.0, -1.0, 1.5, 0.0, 0.9])
+    p = torch.softmax(row, 0)
+    logits = row.expand(50, 6).contiguous()
+    want = 6 * float(p[1] + p[3])
+    assert abs(float(R.load_balancing_loss((logits,), 6, 2)) - want) < 1e-6
+    # perfectly balanced routing with uniform-looking probabilities gives K (the minimum N * K/N * 1/N * N)
+    N, K, T = 8, 2, 64
+    logits = torch.full((T, N), -10.0)
+    for t in range(T):
+        logits[t, t % N] = 1.0; logits[t, (t + 1) % N] = 0.5
+    loss = float(R.load_balancing_loss((logits,), N, K))
+    assert abs(loss - K) < 1e-3
