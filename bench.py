@@ -309,10 +309,12 @@ def main():
                                "2048, 64 experts, top-8, ffn 1024, fp32 router logits, no dropping"},
         "roofline": moe["roofline"], "kernels": moe["kernels"],
     }
+    # GPU workloads first, back to back: the seconds of CPU baseline in between would let the GPU
+    # fall into its idle power state right before the HBM-bound measurement
+    ad = None if args.skip_adamw else bench_adamw(args, device)
     if not args.skip_cpu:
         out["cpu_baseline"] = cpu_baseline_moe()
-    if not args.skip_adamw:
-        ad = bench_adamw(args, device)
+    if ad is not None:
         if not args.skip_cpu and "skipped" not in ad:
             ad["cpu_baseline"] = cpu_baseline_adamw()
         out["adamw"] = ad
