@@ -46,22 +46,51 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
     T *dst = out + t * E;
     constexpr int V = Elem<T>::VEC;
     if (vec_ok) {
+        // The token's row numbers and weights are fetched once, 64 at a time, one per lane, and
+        // handed round with lane reads: the row loads then depend on no other load, and the four
+        // column chunks a lane owns (4 KB of a row per pass) are in flight together.
+        constexpr int CH = 4;
         const int64_t nv = E / V;
-        for (int64_t c = lane; c < nv; c += 64) {
-            float acc[V];
+        for (int64_t c0 = 0; c0 < nv; c0 += 64 * CH) {
+            float acc[CH][V];
 #pragma unroll
-            for (int j = 0; j < V; j++) acc[j] = 0.0f;
-            for (int32_t i = i0; i < i1; i++) {
-                const int32_t index = output_indices[i];
-                float scaling = 1.0f;
-                if (SCALE) scaling = Elem<TW>::load(routing_weights + t * K + selected_experts_indices[i]);
-                const u32x4 q = reinterpret_cast<const u32x4 *>(rows + static_cast<int64_t>(index) * E)[c];
-                float f[V];
-                Elem<T>::unpack(q, f);
+            for (int u = 0; u < CH; u++)
 #pragma unroll
-                for (int j = 0; j < V; j++) acc[j] += SCALE ? (f[j] * scaling) : f[j];
+                for (int j = 0; j < V; j++) acc[u][j] = 0.0f;
+            for (int32_t ib = i0; ib < i1; ib += 64) {
+                const int32_t n = min(64, i1 - ib);
+                int32_t my_index = 0;
+                float my_scale = 1.0f;
+                if (lane < n) {
+                    my_index = output_indices[ib + lane];
+                    if (SCALE) my_scale = Elem<TW>::load(routing_weights + t * K + selected_experts_indices[ib + lane]);
+                }
+                for (int32_t i = 0; i < n; i++) {
+                    const int32_t index = __shfl(my_index, i, 64);
+                    const float scaling = __shfl(my_scale, i, 64);
+                    const u32x4 *src = reinterpret_cast<const u32x4 *>(rows + static_cast<int64_t>(index) * E);
+                    u32x4 q[CH];
+#pragma unroll
+                    for (int u = 0; u < CH; u++) {
+                        const int64_t c = c0 + u * 64 + lane;
+                        if (c < nv) q[u] = src[c];
+                    }
+#pragma unroll
+                    for (int u = 0; u < CH; u++) {
+                        if (c0 + u * 64 + lane < nv) {
+                            float f[V];
+                            Elem<T>::unpack(q[u], f);
+#pragma unroll
+                            for (int j = 0; j < V; j++) acc[u][j] += SCALE ? (f[j] * scaling) : f[j];
+                        }
+                    }
+                }
             }
-            reinterpret_cast<u32x4 *>(dst)[c] = Elem<T>::pack(acc);
+#pragma unroll
+            for (int u = 0; u < CH; u++) {
+                const int64_t c = c0 + u * 64 + lane;
+                if (c < nv) reinterpret_cast<u32x4 *>(dst)[c] = Elem<T>::pack(acc[u]);
+            }
         }
     } else {
         for (int64_t e = lane; e < E; e += 64) {
