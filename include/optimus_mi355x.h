@@ -241,6 +241,25 @@ int om_reduce_ggemm_output_backward(const void *final_hidden_states_grad, const 
                                     void *stream);
 
 /* ------------------------------------------------------------------------------------
+ * RMSNorm either side of the MoE block, optionally fused with the residual add before it
+ * replaces: OlmoeParallelRMSNorm.forward, optimus/models/olmoe/modeling_olmoe.py:98-104
+ *   (= DeepseekV3ParallelRMSNorm.forward, optimus/models/deepseek_v3/modeling_deepseek_v3.py:35-40)
+ *   and, with `residual`, the add of the decoder layer body in front of it (modeling_olmoe.py:402,
+ *   :405-409): h = x + residual (rounded to the model dtype); r = rsqrt(mean(float(h)^2) + eps);
+ *   out = weight * cast(float(h) * r).  residual, h_out and rstd_out may be NULL (h_out receives h,
+ *   the next residual; rstd_out [rows] fp32 is what the backward needs).  x, residual, weight,
+ *   out, h_out share `dtype`; E a multiple of 8 (bf16) / 4 (fp32); rows of any length.
+ * om_rmsnorm_bwd: dx [rows,E] = r * (g*w - xn * mean(g*w*xn)), xn = float(h)*r, g = dy, and
+ *   dweight [E] = sum_rows dy * cast(xn) (fp32 accumulation, deterministic order), from h (the
+ *   tensor that was normalised) and rstd.  workspace: om_rmsnorm_bwd_workspace_bytes.        */
+int om_rmsnorm_fwd(const void *x, const void *residual, const void *weight, double eps, void *out,
+                   void *h_out, float *rstd_out, int64_t rows, int64_t E, int dtype, void *stream);
+int64_t om_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t E);
+int om_rmsnorm_bwd(const void *dy, const void *h, const void *weight, const float *rstd, void *dx,
+                   void *dweight, void *workspace, int64_t workspace_bytes, int64_t rows, int64_t E,
+                   int dtype, void *stream);
+
+/* ------------------------------------------------------------------------------------
  * Grouped expert GEMMs (bf16 operands, fp32 MFMA accumulation, bf16 results)
  * The G experts own the row segments [cum_token_counts[g], cum_token_counts[g+1]) of the
  * activation matrices; cum_token_counts [G+1] is a DEVICE int32 array (no host copy, no

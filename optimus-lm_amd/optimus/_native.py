@@ -44,6 +44,11 @@ SIGNATURES = {
     "om_router_balance_stats": (c_int, [c_void_p, c_int, c_i64, c_int, c_int, c_void_p, c_void_p,
                                         c_void_p, c_i64, c_void_p]),
     "om_router_balance_bwd": (c_int, [c_void_p, c_int, c_void_p, c_i64, c_int, c_void_p, c_void_p]),
+    "om_rmsnorm_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_double, c_void_p, c_void_p, c_void_p,
+                               c_i64, c_i64, c_int, c_void_p]),
+    "om_rmsnorm_bwd_workspace_bytes": (c_i64, [c_i64, c_i64]),
+    "om_rmsnorm_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_i64, c_i64, c_i64, c_int, c_void_p]),
     "om_route_sigmoid_group_topk": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_int, c_int,
                                             c_int, c_double, c_void_p, c_void_p, c_void_p]),
     "om_route_sigmoid_topk_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int, c_int,
@@ -89,7 +94,7 @@ _lib = None
 # kernel durations from HIP events inside the timed region; None (the default) costs one test.
 launch_log = None
 _UNTIMED = {"om_version", "om_arch", "om_strerror", "om_moe_sort_workspace_bytes",
-            "om_router_balance_workspace_bytes"}
+            "om_router_balance_workspace_bytes", "om_rmsnorm_bwd_workspace_bytes"}
 
 
 class NativeLibraryError(RuntimeError):

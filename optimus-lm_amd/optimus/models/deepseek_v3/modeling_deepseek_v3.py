@@ -17,6 +17,7 @@ from torch.utils.checkpoint import checkpoint as torch_activation_checkpoint
 
 from optimus import _native as _n
 from optimus.models.common import moe as _moe
+from optimus.models.common.norm import ParallelRMSNorm
 
 
 class DeepseekV3ParallelMLP(nn.Module):
@@ -167,3 +168,11 @@ class DeepseekV3ParallelMoE(nn.Module):
             self.experts[local_expert_idx].load_state_dict(
                 module.experts[self.expert_start_idx + local_expert_idx].state_dict())
         self.shared_experts.load_state_dict(module.shared_experts.state_dict())
+
+
+class DeepseekV3ParallelRMSNorm(ParallelRMSNorm):
+    """Reference modeling_deepseek_v3.py:29-44 (eps default 1e-6)."""
+
+    def __init__(self, hidden_size, eps=1e-6):
+        super().__init__(hidden_size, eps)
+

@@ -14,6 +14,7 @@ import torch.nn as nn
 from torch.utils.checkpoint import checkpoint as torch_activation_checkpoint
 
 from optimus.models.common import moe as _moe
+from optimus.models.common.norm import ParallelRMSNorm
 from optimus.models.common.ral_functions import (  # noqa: F401  (same names as the reference module)
     layer_level_load_balancing_loss_func, load_balancing_loss_func)
 
@@ -107,3 +108,11 @@ class OlmoeParallelSparseMoeBlock(nn.Module):
         for local_expert_idx in range(self.num_experts_per_rank):
             self.experts[local_expert_idx].load_state_dict(
                 module.experts[self.expert_start_idx + local_expert_idx].state_dict())
+
+
+class OlmoeParallelRMSNorm(ParallelRMSNorm):
+    """Reference modeling_olmoe.py:93-104 (eps default 1e-5)."""
+
+    def __init__(self, hidden_size, eps=1e-5):
+        super().__init__(hidden_size, eps)
+

@@ -139,3 +139,15 @@ def fast_block_restatement(hidden_states, routing_weights, selected_experts, w_g
                                          idx["selected_experts_indices"], idx["output_indices"]), dt)
     idx.update(ggemm_input=ggemm_input, g=g, u=u, h=h, ggemm_output=y)
     return final, idx
+
+
+def rmsnorm(hidden_states, weight, eps, residual=None):
+    """OlmoeParallelRMSNorm.forward, optimus/models/olmoe/modeling_olmoe.py:98-104, preceded by the
+    residual add of the layer body (:402) when `residual` is given.  Returns (y, h)."""
+    if residual is not None:
+        hidden_states = hidden_states + residual                                   # :402
+    input_dtype = hidden_states.dtype
+    h32 = hidden_states.to(torch.float32)                                          # :100
+    variance = h32.pow(2).mean(-1, keepdim=True)                                   # :101
+    h32 = h32 * torch.rsqrt(variance + eps)                                        # :102
+    return weight * h32.to(input_dtype), hidden_states                             # :103

@@ -79,6 +79,22 @@ def test_sort_and_index_ops(lib):
     assert lib.om_swiglu_bwd(P, P, P, None, P, 64, BF16, None) == NULL
 
 
+def test_rmsnorm_and_balance(lib):
+    assert lib.om_rmsnorm_fwd(P, None, P, 1e-5, P, None, None, 8, 2048, 3, None) == DTYPE
+    assert lib.om_rmsnorm_fwd(P, None, P, 1e-5, P, None, None, 8, 2052, BF16, None) == SHAPE   # E % 8
+    assert lib.om_rmsnorm_fwd(P, None, P, 1e-5, P, None, None, 0, 2048, BF16, None) == OK
+    assert lib.om_rmsnorm_fwd(P, None, None, 1e-5, P, None, None, 8, 2048, BF16, None) == NULL
+    assert lib.om_rmsnorm_fwd(P, ODD, P, 1e-5, P, None, None, 8, 2048, BF16, None) == ALIGN
+    need = lib.om_rmsnorm_bwd_workspace_bytes(300, 2048)
+    assert need == 3 * 2048 * 4
+    assert lib.om_rmsnorm_bwd(P, P, P, P, P, P, P, need - 1, 300, 2048, BF16, None) == WORKSPACE
+    assert lib.om_rmsnorm_bwd(P, P, P, None, P, P, P, need, 300, 2048, BF16, None) == NULL
+    need = lib.om_router_balance_workspace_bytes(1000, 64)
+    assert lib.om_router_balance_stats(P, F32, 1000, 64, 8, P, P, P, need - 1, None) == WORKSPACE
+    assert lib.om_router_balance_stats(P, 9, 1000, 64, 8, P, P, P, need, None) == DTYPE
+    assert lib.om_router_balance_bwd(P, F32, None, 1000, 64, P, None) == NULL
+
+
 def test_grouped_gemms(lib):
     args = (131072, 64, 2048, 1024, 0, None)
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 131072, 64, 2000, 1024, 0, None) == SHAPE    # N % 128
