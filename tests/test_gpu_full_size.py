@@ -89,3 +89,48 @@ def test_c3_full_size_index_construction(cuda):
     same = row_expert[1:] == row_expert[:-1]
     assert bool((ii[1:][same] > ii[:-1][same]).all())
     assert torch.equal(cum_ep.cpu().long(), torch.arange(T + 1) * K)
+
+
+def test_c5_full_size_one_rank_share(cuda):
+    """C5 at its real shape: 8192 tokens, hidden 7168, this rank's 32 of 256 routed experts (ffn 2048)
+    plus the shared expert.  Same properties: determinism, permutation, exact scaling."""
+    from optimus.mapper import ParallelDpPpEpTpMapper
+    from optimus.models.deepseek_v3.configuration_deepseek_v3 import DeepseekV3ParallelConfig
+    from optimus.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3ParallelMoE
+    inp = sc.dsv3_inputs()
+    c = inp["cfg"]
+    T, H = c["T"], c["H"]
+    cfg = DeepseekV3ParallelConfig(expert_parallelism=8)
+    assert (cfg.hidden_size, cfg.moe_intermediate_size, cfg.n_routed_experts) == (H, c["I"], c["N"])
+    blk = DeepseekV3ParallelMoE(cfg, ParallelDpPpEpTpMapper(expert_parallelism=8, rank=2)).to(cuda).to(torch.bfloat16)
+    with torch.no_grad():
+        blk.gate.weight.copy_(inp["router_w"]); blk.gate.e_score_correction_bias.copy_(inp["bias"])
+        for e, m in enumerate(blk.experts):
+            m.gate_proj.weight.copy_(inp["w_gate"][e]); m.up_proj.weight.copy_(inp["w_up"][e])
+            m.down_proj.weight.copy_(inp["w_down"][e])
+        blk.shared_experts.gate_proj.weight.copy_(inp["ws_gate"]); blk.shared_experts.up_proj.weight.copy_(inp["ws_up"])
+        blk.shared_experts.down_proj.weight.copy_(inp["ws_down"])
+    x = inp["x"].to(cuda); dout = inp["dout"].to(cuda)
+
+    def run(xx, dd):
+        for p in blk.parameters():
+            p.grad = None
+        xg = xx.clone().requires_grad_(True)
+        out = blk(xg.view(2, T // 2, H))
+        out.backward(dd.view_as(out))
+        return out.detach().reshape(T, H), xg.grad.clone()
+
+    out, dx = run(x, dout)
+    e, w = blk.gate(x)
+    local = ((e >= 64) & (e < 96)).sum()
+    assert torch.isfinite(out.float()).all() and int(local) > 0.8 * T      # about T routed rows on this rank
+    out_r, dx_r = run(x, dout)
+    assert torch.equal(out_r, out) and torch.equal(dx_r, dx)
+    perm = torch.randperm(T, generator=torch.Generator().manual_seed(6)).to(cuda)
+    out_p, dx_p = run(x[perm], dout[perm])
+    for got, want in ((out_p, out[perm]), (dx_p, dx[perm])):
+        d = (got.float() - want.float()).abs()
+        assert float((d > 0).float().mean()) <= 0.05
+        assert float(d.max()) <= 2.0 ** -6 * float(want.float().abs().max())
+    out_2, dx_2 = run(x, dout * 2)
+    assert torch.equal(out_2, out) and torch.equal(dx_2, dx * 2)
