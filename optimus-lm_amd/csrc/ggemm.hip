@@ -18,9 +18,10 @@
 // choosing which global chunk each lane fetches.  The per-lane order of the 8 contraction
 // indices is the same for both kinds, so they can be mixed in one MFMA.
 //
-// Variable rows per expert: the M extent of fwd/dgrad is cut into tiles per expert; a block finds
-// its (expert, row block) from the device-resident cum_token_counts with a wavefront scan, so no
-// host copy of the counts and no max-rows-per-expert is needed.  In wgrad the rows are the
+// Variable rows per expert: the M extent of fwd/dgrad is cut into tiles per expert.  Each block
+// scans the device-resident cum_token_counts once into an LDS table (row tiles up to and including
+// each expert) and looks its (expert, row block) up there per tile, so no host copy of the counts
+// and no max-rows-per-expert is needed, and the blocks share out the tiles that really exist.  In wgrad the rows are the
 // contraction range of expert g; rows past its end are zero-filled in LDS.
 //
 // Block order: consecutive block ids go to different XCDs (8 per chip, each with its own L2), so
@@ -126,6 +127,13 @@ __device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
+// 1 / (1 + e^-x) with the hardware exponential and reciprocal (about 1 ulp each, far inside one
+// bf16 rounding of the results it feeds).  An IEEE division here costs ten instructions per
+// element, and the SwiGLU epilogues are bound by vector-ALU issue.
+__device__ __forceinline__ float fast_sigmoid(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
+
 __device__ __forceinline__ void unpack4_bf16(u32x2 v, float *f) {
     f[0] = __uint_as_float(v[0] << 16);
     f[1] = __uint_as_float(v[0] & 0xffff0000u);
@@ -133,36 +141,47 @@ __device__ __forceinline__ void unpack4_bf16(u32x2 v, float *f) {
     f[3] = __uint_as_float(v[1] & 0xffff0000u);
 }
 
-// Which expert owns row tile `tile` (tiles are BM rows, cut per expert)?  Wavefront scan over
-// cum_token_counts.  Returns false when `tile` is past the last tile.
+// Row tiles of fwd/dgrad are cut per expert (BM rows each, the last one of an expert partial).
+// One wavefront builds, once per block, a table in LDS from the device-resident cum_token_counts:
+// tile_end[e] = number of row tiles of experts 0..e, seg[e] = cum_token_counts[e].
+constexpr int MAX_EXPERTS = 1024;
 template <int BM>
-__device__ __forceinline__ bool find_tile(const int32_t *cum, int n_experts, int tile, int lane,
-                                          int &expert, int &row_begin, int &row_end) {
+__device__ __forceinline__ void build_tile_table(const int32_t *cum, int n_experts, int lane,
+                                                 int *tile_end, int *seg) {
     int base_tiles = 0;
     for (int e0 = 0; e0 < n_experts; e0 += 64) {
         const int e = e0 + lane;
         int s = 0, cnt = 0;
         if (e < n_experts) { s = cum[e]; cnt = cum[e + 1] - s; }
-        const int tiles = (cnt + BM - 1) / BM;
-        int incl = tiles;  // inclusive scan over the wavefront
+        int incl = (cnt + BM - 1) / BM;  // inclusive scan over the wavefront
         for (int o = 1; o < 64; o <<= 1) {
             const int v = __shfl_up(incl, o, 64);
             if (lane >= o) incl += v;
         }
-        const int excl = incl - tiles;
-        const bool mine = (tile >= base_tiles + excl) && (tile < base_tiles + incl);
-        const unsigned long long vote = __ballot(mine);
-        if (vote) {
-            const int src = __ffsll(static_cast<long long>(vote)) - 1;
-            const int local = tile - (base_tiles + __shfl(excl, src, 64));
-            const int s_src = __shfl(s, src, 64);
-            const int cnt_src = __shfl(cnt, src, 64);
-            expert = e0 + src;
-            row_begin = s_src + local * BM;
-            row_end = s_src + cnt_src;
-            return true;
+        if (e < n_experts) {
+            tile_end[e] = base_tiles + incl;
+            seg[e] = s;
+            if (e == n_experts - 1) seg[n_experts] = s + cnt;
         }
         base_tiles += __shfl(incl, 63, 64);
+    }
+}
+
+// Which expert owns row tile `tile`, and which rows are the tile's?  False past the last tile.
+template <int BM>
+__device__ __forceinline__ bool find_tile(const int *tile_end, const int *seg, int n_experts, int tile,
+                                          int lane, int &expert, int &row_begin, int &row_end) {
+    for (int e0 = 0; e0 < n_experts; e0 += 64) {
+        const int e = e0 + lane;
+        const bool mine = e < n_experts && tile < tile_end[e];   // tile_end is non-decreasing
+        const unsigned long long vote = __ballot(mine);
+        if (vote) {
+            expert = e0 + __ffsll(static_cast<long long>(vote)) - 1;
+            const int first = expert > 0 ? tile_end[expert - 1] : 0;
+            row_begin = seg[expert] + (tile - first) * BM;
+            row_end = seg[expert + 1];
+            return true;
+        }
     }
     return false;
 }
@@ -181,6 +200,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // stage does not depend on the loads in flight to the other
     __shared__ __attribute__((aligned(1024))) char stage0[A_BYTES + B_BYTES];
     __shared__ __attribute__((aligned(1024))) char stage1[A_BYTES + B_BYTES];
+    __shared__ int tile_end[EPI == EPI_WGRAD ? 1 : MAX_EXPERTS];   // see build_tile_table
+    __shared__ int seg[EPI == EPI_WGRAD ? 1 : MAX_EXPERTS + 1];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -248,7 +269,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             const int tile_m = logical / tiles_n;
             const int tile_n = logical % tiles_n;
             rot_a = tile_n; rot_b = tile_m & 7;
-            if (!find_tile<BM>(p.cum, p.n_experts, tile_m, lane_s, expert, row_begin, row_end)) return false;
+            if (!find_tile<BM>(tile_end, seg, p.n_experts, tile_m, lane_s, expert, row_begin, row_end)) return false;
             n0 = tile_n * BN_OUT;
             c_begin = 0;
             c_len = p.kc;
@@ -495,9 +516,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // tiles and its blocks take them round-robin, so the tiles in flight on an XCD at any moment
     // are neighbours and share operand slices in that XCD's L2; the total % 8 tiles left over go
     // one each to the blocks of the least loaded slot.
+    // fwd/dgrad: the launch is sized for an upper bound on the row tiles; the tiles that exist are
+    // counted here from cum_token_counts, so that all XCDs get equal shares of real work.
+    int total_tiles = p.total_tiles;
+    if (EPI != EPI_WGRAD) {
+        if (wave == 0) build_tile_table<BM>(p.cum, p.n_experts, lane, tile_end, seg);
+        __syncthreads();
+        constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
+        total_tiles = __builtin_amdgcn_readfirstlane(tile_end[p.n_experts - 1]) * (p.n_cols / BN_OUT);
+    }
     const int nbx = gridDim.x / NUM_XCD;
     const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
-    const int per = p.total_tiles / NUM_XCD, rem = p.total_tiles - per * NUM_XCD;
+    const int per = total_tiles / NUM_XCD, rem = total_tiles - per * NUM_XCD;
     const int n_mine = slot < per ? (per - slot + nbx - 1) / nbx : 0;
     const int n_all = n_mine + ((xcd < rem && slot == per % nbx) ? 1 : 0);
     int it = 0;
@@ -600,7 +630,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 #pragma unroll
                     for (int x = 0; x < 4; x++) {
                         const float gv = acc[i][j][rq * 4 + x], uv = acc[i][j + 1][rq * 4 + x];
-                        hv[x] = (gv / (1.0f + __expf(-gv))) * uv;
+                        hv[x] = (gv * fast_sigmoid(gv)) * uv;
                     }
                     const int col = (j / 2) * 32 + rq * 8 + lcol;
                     strip_put(0, col, acc[i][j][rq * 4], acc[i][j][rq * 4 + 1], acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3]);
@@ -639,7 +669,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                     Elem<uint16_t>::unpack(uq[it], uv);
 #pragma unroll
                     for (int x = 0; x < 8; x++) {
-                        const float sg = 1.0f / (1.0f + __expf(-gv[x]));
+                        const float sg = fast_sigmoid(gv[x]);
                         du[x] = dh[x] * (gv[x] * sg);
                         dg[x] = (dh[x] * uv[x]) * (sg * (1.0f + gv[x] * (1.0f - sg)));
                     }
@@ -711,6 +741,7 @@ template <int BM> struct Waves {
 template <int BM, int BN, int AKIND, int BKIND, int EPI>
 int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad family
     constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
+    if (p.n_experts > MAX_EXPERTS) return OM_ERR_SHAPE;   // the tile table lives in LDS
     p.m_tiles_max = static_cast<int>((rows + BM - 1) / BM + p.n_experts);
     const int64_t tiles = static_cast<int64_t>(p.m_tiles_max) * (p.n_cols / BN_OUT);
     if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
