@@ -131,6 +131,21 @@ int om_router_gate_softmax_topk(const void *x, const void *gate_weight, int64_t 
 int om_router_gate_logits(const void *x, const void *gate_weight, int64_t T, int H, int N,
                           float *logits_out, void *stream);
 
+/* om_router_gate_wgrad: gradient of the gate's weight,
+ *   dweight[n,h] = sum_t dlogits[t,n] * x[t,h]
+ * i.e. what autograd computes for the nn.Linear behind `router_logits = self.gate(hidden_states)`
+ * (optimus/models/common/moe.py:456, optimus/models/olmoe/modeling_olmoe.py:284) from the
+ * gradient of the logits.  x [T,H] bf16; dlogits [T,N] fp32, rounded to bf16 as it is loaded;
+ * products accumulate in fp32 over token ranges and the partial sums are added in a fixed order
+ * (deterministic).  dweight [N,H] in dweight_dtype (OM_BF16 / OM_F32).  N in {32,64,128,256},
+ * H a multiple of 128; other shapes return OM_ERR_SHAPE and the caller uses a library GEMM.
+ * workspace: om_router_gate_wgrad_workspace_bytes(T,H,N) bytes of device memory, 16-byte
+ * aligned (negative = error code).                                                        */
+int64_t om_router_gate_wgrad_workspace_bytes(int64_t T, int H, int N);
+int om_router_gate_wgrad(const void *x, const float *dlogits, int64_t T, int H, int N,
+                         void *dweight, int dweight_dtype, void *workspace,
+                         int64_t workspace_bytes, void *stream);
+
 /* Load-balancing statistics of one layer's router logits
  * replaces: the per-token part of load_balancing_loss_func,
  *   optimus/models/olmoe/modeling_olmoe.py:44-57 (softmax, top-K, one-hot mean, probability
@@ -273,7 +288,9 @@ int om_rmsnorm_bwd(const void *dy, const void *h, const void *weight, const floa
  * w_stride: elements between the matrices of consecutive experts in `weight` /
  * `weight_grad`; 0 means densely packed (N*K, the merged [G,N,K] layout).  A larger stride
  * serves per-expert nn.Linear weights that sit at a constant pitch inside one flat buffer.
- * N and K must be multiples of 128.                                                       */
+ * N and K must be multiples of 128.  fwd and dgrad (and the merged-MLP fusions below) keep
+ * a per-expert tile table in LDS and take G <= 1024 (OM_ERR_SHAPE above that); wgrad has no
+ * such limit.                                                                             */
 int om_grouped_gemm_fwd(const void *input, const void *weight, void *output,
                         const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                         int64_t w_stride, void *stream);

@@ -90,13 +90,44 @@ def gate_kernel_fits(x, weight):
     return H % (512 if N <= 64 else 256 if N <= 128 else 64) == 0
 
 
+def gate_wgrad_kernel_fits(x, weight):
+    """Shapes om_router_gate_wgrad takes."""
+    N, H = weight.shape
+    return (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype in (torch.bfloat16, torch.float32)
+            and N in (32, 64, 128, 256) and H % 128 == 0)
+
+
+def _gate_weight_grad(x, weight, dlogits):
+    """dweight[n,h] = sum_t dlogits[t,n] x[t,h]: a long contraction with a tiny output, split
+    over token ranges on the device (om_router_gate_wgrad) instead of a library GEMM that would
+    run on a few CUs."""
+    T, (N, H) = x.shape[0], weight.shape
+    lib = _n.lib()
+    ws_bytes = lib.om_router_gate_wgrad_workspace_bytes(T, H, N)
+    if ws_bytes < 0:
+        _n.check(int(ws_bytes), "om_router_gate_wgrad_workspace_bytes")
+    workspace = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=x.device)
+    dw = torch.empty_like(weight)
+    dlogits = dlogits.contiguous()
+    _n.check(lib.om_router_gate_wgrad(_n.ptr(x), _n.ptr(dlogits), T, H, N, _n.ptr(dw), _n.dtype_code(dw),
+                                      _n.ptr(workspace), int(ws_bytes), _n.stream()),
+             "om_router_gate_wgrad")
+    return dw
+
+
 def _gate_backward(x, weight, dlogits, needs):
-    """(dx, dweight) of logits = x @ weight.T from the fp32 gradient of the logits: rounded to bf16
-    (the precision a bf16 router's backward has anyway), two library GEMMs, the weight gradient
-    accumulated in fp32."""
-    d16 = dlogits.to(torch.bfloat16)
-    dx = torch.mm(d16, weight) if needs[0] else None
-    dw = torch.mm(d16.t(), x, out_dtype=torch.float32).to(weight.dtype) if needs[1] else None
+    """(dx, dweight) of logits = x @ weight.T from the fp32 gradient of the logits, rounded to
+    bf16 (the precision a bf16 router's backward has anyway): dx by a library GEMM, the weight
+    gradient accumulated in fp32 by om_router_gate_wgrad (a library GEMM for shapes it does not
+    take)."""
+    dx = dw = None
+    if needs[0]:
+        dx = torch.mm(dlogits.to(torch.bfloat16), weight)
+    if needs[1]:
+        if gate_wgrad_kernel_fits(x, weight) and dlogits.dtype == torch.float32:
+            dw = _gate_weight_grad(x, weight, dlogits)
+        else:
+            dw = torch.mm(dlogits.to(torch.bfloat16).t(), x, out_dtype=torch.float32).to(weight.dtype)
     return dx, dw
 
 

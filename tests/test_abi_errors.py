@@ -61,6 +61,16 @@ def test_routers(lib):
     assert lib.om_router_gate_softmax_topk(ODD, P, 8, 2048, 64, 8, 0, P, P, BF16, P, None) == ALIGN
     assert lib.om_router_gate_softmax_topk(P, P, 8, 2048, 64, 8, 0, P, None, BF16, P, None) == NULL
     assert lib.om_router_gate_logits(P, P, 8, 2048, 64, None, None) == NULL
+    need = lib.om_router_gate_wgrad_workspace_bytes(16384, 2048, 64)
+    assert need > 0 and need % 16 == 0
+    assert lib.om_router_gate_wgrad_workspace_bytes(16384, 2000, 64) == SHAPE      # H % 128
+    assert lib.om_router_gate_wgrad_workspace_bytes(16384, 2048, 48) == SHAPE      # N not 32/64/128/256
+    assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 64, P, 7, P, need, None) == DTYPE
+    assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 96, P, BF16, P, need, None) == SHAPE
+    assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 64, None, BF16, P, need, None) == NULL
+    assert lib.om_router_gate_wgrad(P, None, 16384, 2048, 64, P, BF16, P, need, None) == NULL
+    assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 64, ODD, BF16, P, need, None) == ALIGN
+    assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 64, P, BF16, P, need - 1, None) == WORKSPACE
 
 
 def test_sort_and_index_ops(lib):
@@ -99,6 +109,7 @@ def test_grouped_gemms(lib):
     args = (131072, 64, 2048, 1024, 0, None)
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 131072, 64, 2000, 1024, 0, None) == SHAPE    # N % 128
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 0, 64, 2048, 1024, 0, None) == OK            # no rows
+    assert lib.om_grouped_gemm_fwd(P, P, P, P, 4096, 1025, 256, 256, 0, None) == SHAPE      # G > 1024 (LDS table)
     assert lib.om_grouped_gemm_fwd(P, None, P, P, *args) == NULL
     assert lib.om_grouped_gemm_fwd(P, P, ODD, P, *args) == ALIGN
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 1 << 22, 64, 2048, 1024, 0, None) == SHAPE   # > 2^31 elements

@@ -43,7 +43,10 @@ def _ref_fwd(x, w, cum):
 CASES = [("uniform", 4, 512, 256, 128), ("ragged", 8, 1000, 256, 512), ("empties", 16, 777, 128, 256),
          ("ragged", 64, 4096, 1024, 2048), ("uniform", 1, 300, 256, 256), ("ragged", 3, 5, 128, 128),
          # several tiles per persistent block, on both tile shapes, with empty experts in between
-         ("ragged", 8, 20000, 512, 768), ("ragged", 8, 20000, 384, 640), ("empties", 32, 9000, 512, 1024)]
+         ("ragged", 8, 20000, 512, 768), ("ragged", 8, 20000, 384, 640), ("empties", 32, 9000, 512, 1024),
+         # more experts than lanes in a wavefront: the per-block tile table is built in several
+         # rounds with a carry, the last one partial
+         ("ragged", 150, 6000, 128, 128), ("empties", 200, 70000, 256, 256)]
 
 
 @pytest.mark.parametrize("kind,G,rows,N,K", CASES)

@@ -210,6 +210,34 @@ def test_gate_softmax_topk_backward(cuda):
     assert not torch.equal(gx1, xg.grad)     # the logits' own gradient takes part
 
 
+@pytest.mark.parametrize("T,H,N,wdt", [(16384, 2048, 64, torch.bfloat16), (1, 128, 32, torch.float32),
+                                       (100, 256, 64, torch.float32), (5000, 1024, 128, torch.bfloat16),
+                                       (777, 7168, 256, torch.float32), (64, 2048, 64, torch.float32)])
+def test_gate_weight_grad_matches_fp32_matmul(cuda, T, H, N, wdt):
+    """om_router_gate_wgrad against the product it replaces: dlogits rounded to bf16, multiplied in
+    fp32.  The bf16 x bf16 products are exact in fp32, so only the order of the fp32 sum differs
+    (float64 reference; bound = a few fp32 roundings of the absolute sum), plus one final rounding
+    for a bf16 weight.  Token counts that are not multiples of the 64-token stage or of the split."""
+    from optimus.models.common.moe import _gate_weight_grad, gate_wgrad_kernel_fits
+    g = torch.Generator().manual_seed(T + N)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    dl = torch.randn(T, N, generator=g) * 0.3
+    w = torch.empty(N, H, dtype=wdt)
+    assert gate_wgrad_kernel_fits(x.to(cuda), w.to(cuda))
+    out = _gate_weight_grad(x.to(cuda), w.to(cuda), dl.to(cuda))
+    assert out.dtype == wdt and out.shape == (N, H)
+    d16 = dl.to(torch.bfloat16).double()
+    ref = d16.t() @ x.double()
+    bound = 1e-6 * (d16.abs().t() @ x.double().abs()) + 1e-30
+    err = (out.double().cpu() - ref).abs()
+    if wdt == torch.bfloat16:
+        bound = bound + ref.abs() * 2.0 ** -8      # one bf16 rounding
+    assert bool((err <= bound).all()), float((err / bound).max())
+    # deterministic: same bits on a second run
+    out2 = _gate_weight_grad(x.to(cuda), w.to(cuda), dl.to(cuda))
+    assert torch.equal(out, out2)
+
+
 # ---- auxiliary load-balancing loss (om_router_balance_stats / _bwd) ---------------------------------
 @pytest.mark.parametrize("L,T,N,K", [(3, 4096, 64, 8), (2, 1000, 100, 5), (1, 77, 256, 8), (4, 512, 8, 2)])
 def test_balance_losses_match_the_reference_expressions(cuda, L, T, N, K):
