@@ -96,6 +96,7 @@ _lib = None
 # appends (name, start_event, end_event) recorded on the current stream.  Used by bench.py to get
 # kernel durations from HIP events inside the timed region; None (the default) costs one test.
 launch_log = None
+launch_filter = None   # optional set of entry-point names: only these are timed while launch_log is set
 _UNTIMED = {"om_version", "om_arch", "om_strerror", "om_moe_sort_workspace_bytes",
             "om_router_balance_workspace_bytes", "om_rmsnorm_bwd_workspace_bytes",
             "om_router_gate_wgrad_workspace_bytes"}
@@ -118,7 +119,7 @@ class _Library:
     @staticmethod
     def _maybe_timed(name, fn):
         def call(*args):
-            if launch_log is None:
+            if launch_log is None or (launch_filter is not None and name not in launch_filter):
                 return fn(*args)
             a = torch.cuda.Event(enable_timing=True)
             b = torch.cuda.Event(enable_timing=True)
