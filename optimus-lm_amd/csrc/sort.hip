@@ -2,7 +2,7 @@
 // local expert, producing exactly the arrays the reference builds with its two index kernels and
 // two cumsums.  Three small launches:
 //   count   — every block histograms its chunk of pairs per expert (wave ballots -> LDS);
-//   scan    — one block turns the [block][expert] table into exclusive offsets in
+//   scan    — one block (16 wavefront-wide scans at a time) turns the [block][expert] table into exclusive offsets in
 //             (expert-major, block-minor) order = the stable order, and writes cum_token_counts;
 //   scatter — every block re-reads its chunk and places each pair at offset + stable rank.
 // Ranks come from wavefront ballots (lanes holding the same expert form a mask; rank = popcount of
@@ -76,49 +76,72 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_count_kernel(const TI *__re
     }
 }
 
+// Inclusive prefix sum over the 64 lanes of a wavefront.
+__device__ __forceinline__ int wave_incl_scan(int v, int lane) {
+    for (int o = 1; o < 64; o <<= 1) {
+        const int u = __shfl_up(v, o, 64);
+        if (lane >= o) v += u;
+    }
+    return v;
+}
+
 // One block.  block_hist [NB][NR] -> in place: exclusive offset of (expert e, block b) in the
 // stable order; hits_base [NB] = pairs kept by blocks before b; cum_token_counts [NR+1].
+// Every phase is spread over the 16 wavefronts (lanes over blocks or over experts, wavefront
+// scans), so nothing walks the table serially.
 __global__ __launch_bounds__(1024) void sort_scan_kernel(int32_t *__restrict__ block_hist,
                                                           int32_t *__restrict__ hits_base, int NB,
                                                           int NR, int32_t *__restrict__ cum_token_counts,
                                                           int32_t *__restrict__ cum_expert_counts_ep,
                                                           int64_t T) {
     __shared__ int totals[SORT_MAX_NR + 1];
-    // per-expert exclusive scan over blocks
-    for (int e = threadIdx.x; e < NR; e += blockDim.x) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    // per-expert exclusive scan over blocks: one wavefront per expert, lanes over blocks
+    for (int e = wv; e < NR; e += n_waves) {
         int run = 0;
-        for (int b = 0; b < NB; b++) {
-            const int c = block_hist[static_cast<int64_t>(b) * NR + e];
-            block_hist[static_cast<int64_t>(b) * NR + e] = run;
-            run += c;
+        for (int b0 = 0; b0 < NB; b0 += 64) {
+            const int b = b0 + lane;
+            const int c = b < NB ? block_hist[static_cast<int64_t>(b) * NR + e] : 0;
+            const int incl = wave_incl_scan(c, lane);
+            if (b < NB) block_hist[static_cast<int64_t>(b) * NR + e] = run + incl - c;
+            run += __shfl(incl, 63, 64);
         }
-        totals[e] = run;
+        if (lane == 0) totals[e] = run;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {  // NR <= 1024: a serial scan is a microsecond
+    if (wv == 0) {  // exclusive scan of the per-expert totals
         int run = 0;
-        for (int e = 0; e < NR; e++) {
-            const int c = totals[e];
-            totals[e] = run;
-            cum_token_counts[e] = run;
-            run += c;
+        for (int e0 = 0; e0 < NR; e0 += 64) {
+            const int e = e0 + lane;
+            const int c = e < NR ? totals[e] : 0;
+            const int incl = wave_incl_scan(c, lane);
+            if (e < NR) {
+                totals[e] = run + incl - c;
+                cum_token_counts[e] = run + incl - c;
+            }
+            run += __shfl(incl, 63, 64);
         }
-        totals[NR] = run;
-        cum_token_counts[NR] = run;
-        cum_expert_counts_ep[T] = run;
+        if (lane == 0) {
+            totals[NR] = run;
+            cum_token_counts[NR] = run;
+            cum_expert_counts_ep[T] = run;
+        }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < NR; e += blockDim.x) {
-        const int base = totals[e];
-        for (int b = 0; b < NB; b++) block_hist[static_cast<int64_t>(b) * NR + e] += base;
-    }
-    // pairs kept per block = offset(e, b+1) - offset(e, b) summed over e; recompute from the
-    // offsets just written: kept(b) = sum_e (off[b+1][e] - off[b][e]) with off[NB][e] = totals[e+1].
-    __syncthreads();
-    for (int b = threadIdx.x; b < NB; b += blockDim.x) {
-        int kept_before = 0;  // pairs of blocks < b = sum_e (off[b][e] - totals[e])
-        for (int e = 0; e < NR; e++) kept_before += block_hist[static_cast<int64_t>(b) * NR + e] - totals[e];
-        hits_base[b] = kept_before;
+    // add the expert's base, and per block sum what its experts hold before it:
+    // kept_before(b) = sum_e (off[b][e] - totals[e]) = sum_e of the within-expert offsets
+    for (int b = wv; b < NB; b += n_waves) {
+        int kept_before = 0;
+        for (int e0 = 0; e0 < NR; e0 += 64) {
+            const int e = e0 + lane;
+            if (e < NR) {
+                const int within = block_hist[static_cast<int64_t>(b) * NR + e];
+                kept_before += within;
+                block_hist[static_cast<int64_t>(b) * NR + e] = within + totals[e];
+            }
+        }
+        kept_before = wave_sum_i(kept_before);
+        if (lane == 0) hits_base[b] = kept_before;
     }
 }
 

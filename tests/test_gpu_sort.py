@@ -19,6 +19,7 @@ CASES = [
     (1000 * 8, 16, 4, 4, 12, 2.0, torch.int64),    # window + skew
     (24, 64, 8, 0, 64, 3.0, torch.int64),          # tiny T, most experts empty
     (4104, 300, 3, 0, 300, 0.0, torch.int64),      # > 256 experts, pairs not a multiple of 64
+    (40000, 128, 8, 0, 128, 0.5, torch.int64),     # 157 count blocks: the scan walks them 64 at a time
 ]
 
 
