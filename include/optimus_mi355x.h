@@ -321,6 +321,27 @@ int om_merged_mlp_gate_up_dgrad(const void *dg, const void *du, const void *w_ga
                                 int64_t rows, int G, int I, int H, int64_t w_stride,
                                 void *stream);
 
+/* The token gather folded into the GEMMs' operand loads: K4's
+ *   ggemm_input = hidden_states[input_indices]        (PrepareInputForGroupGemmFunction.forward,
+ *   optimus/models/common/moe.py:217-237; index_gather, sparse_moe_block.sycl:56-106)
+ * is never materialised.  The kernels read row input_indices[r] of hidden_states [src_rows, H]
+ * wherever the plain entry points read row r of ggemm_input [rows, H]; the arithmetic, and so
+ * every output bit, is the same as index_gather followed by the plain entry point.
+ *   om_merged_mlp_gate_up_fwd_gathered : as om_merged_mlp_gate_up_fwd with x = hidden_states,
+ *                                        x_rows = input_indices [rows] int32 (device)
+ *   om_grouped_gemm_wgrad_gathered     : as om_grouped_gemm_wgrad with input = hidden_states
+ *                                        [src_rows, K], input_rows = input_indices [rows]
+ *                                        (dW_gate = dg.T @ x[input_indices], same for up)
+ * Indices must lie in [0, src_rows); they are not checked on the device.                   */
+int om_merged_mlp_gate_up_fwd_gathered(const void *x, const int32_t *x_rows, int64_t src_rows,
+                                       const void *w_gate, const void *w_up, void *g, void *u,
+                                       void *h, const int32_t *cum_token_counts, int64_t rows,
+                                       int G, int I, int H, int64_t w_stride, void *stream);
+int om_grouped_gemm_wgrad_gathered(const void *output_grad, const void *input,
+                                   const int32_t *input_rows, int64_t src_rows, void *weight_grad,
+                                   const int32_t *cum_token_counts, int64_t rows, int G, int N,
+                                   int K, int64_t w_stride, void *stream);
+
 /* Stand-alone SwiGLU glue (moe.py:401-402 forward; moe.py:37-41 and :133-147 backward),
  * for callers that keep the three GEMMs separate.  n elements, dtype OM_F32 or OM_BF16.   */
 int om_swiglu_fwd(const void *g, const void *u, void *h, int64_t n, int dtype, void *stream);

@@ -31,6 +31,9 @@
 namespace {
 
 enum { CONTIG = 0, STRIDED = 1 };
+// An operand's rows can be taken through an index instead of in order: the token gather that
+// precedes the expert GEMMs (ggemm_input = hidden_states[input_indices]) folded into the loads.
+enum { GATHER_NONE = 0, GATHER_A = 1 /* fwd: A rows */, GATHER_B = 2 /* wgrad: contraction rows of B */ };
 enum {
     EPI_STORE = 0,        // C = acc
     EPI_SWIGLU = 1,       // even 32-col accumulators = gate, odd = up: store g, u, h
@@ -61,6 +64,7 @@ struct GemmParams {
     const uint16_t *G;   // EPI_SWIGLU_BWD: saved g
     const uint16_t *U;   // EPI_SWIGLU_BWD: saved u
     const int32_t *cum;  // [G+1] device
+    const int32_t *row_index;   // GATHER_A: A row of sorted row r; GATHER_B: B row of contraction row c
     int64_t lda, ldb, ldc;      // leading dimensions, elements
     int64_t strideB, strideC;   // per-expert strides, elements
     int64_t rows;               // allocated activation rows (upper bound of cum[G])
@@ -186,8 +190,10 @@ __device__ __forceinline__ bool find_tile(const int *tile_end, const int *seg, i
     return false;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const GemmParams p) {
+    static_assert(GATHER == GATHER_NONE || (GATHER == GATHER_A && AKIND == CONTIG && EPI != EPI_WGRAD) ||
+                      (GATHER == GATHER_B && BKIND == STRIDED && EPI == EPI_WGRAD), "gather variants");
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
     constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 accumulators per wavefront
@@ -230,6 +236,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     int a_crow[A_LOADS];  // STRIDED A in wgrad: c-row of the lane's slot (for the zero fill)
     int b_crow[B_LOADS];
     bool b_up[B_LOADS];   // EPI_SWIGLU: this LDS row comes from the up matrix
+    int b_src[GATHER == GATHER_B ? B_LOADS : 1];   // GATHER_B: source rows of the next B loads
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
         constexpr int CPR = BM / 8;
@@ -242,6 +249,22 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         b_crow[i] = (BKIND == CONTIG) ? 0 : grp * (64 / CPR) + lane / CPR;
         b_up[i] = (EPI == EPI_SWIGLU) ? (((grp * 8 + (lane >> 3)) >> 5) & 1) : false;
     }
+
+    const int lda32 = static_cast<int>(p.lda), ldb32 = static_cast<int>(p.ldb);
+    // GATHER_B: the B rows that contraction step `step` needs, looked up one step ahead of the
+    // loads that use them (plain loads: they land before the next wait for the direct loads).
+    auto load_b_src = [&](int step) {
+        if (GATHER != GATHER_B || step >= loop_steps) return;
+        const int c0 = (step < steps_per_phase ? rotated(step) : step) * BK;
+        // One 4-byte load per B load (measured faster than one load per wavefront plus lane
+        // permutes, which queue behind the fragment reads).  Kept as loaded: any arithmetic on the
+        // value here would put the wait for the load here too.
+#pragma unroll
+        for (int i = 0; i < B_LOADS; i++) {
+            const int c = min(c0 + b_crow[i], c_len - 1);   // past the segment: any valid row (A is zeroed)
+            b_src[GATHER == GATHER_B ? i : 0] = p.row_index[c_begin + c];
+        }
+    };
 
     // Which tile `logical` is, and the load offsets for it.  False: the tile lies past the last
     // row block (the launch sizes the tile count from an upper bound on the routed rows).
@@ -297,6 +320,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                 const int ch = (lane_s & 7) ^ swz(row);
                 int64_t m = static_cast<int64_t>(row_begin) + row;
                 if (m >= row_end) m = row_end - 1;  // rows past the segment: valid memory, result unused
+                if (GATHER == GATHER_A) m = p.row_index[m];
                 a_off[i] = static_cast<int>(m * p.lda + ch * 8);
             } else {
                 constexpr int CPR = BM / 8;
@@ -324,12 +348,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                 b_off[i] = static_cast<int>((EPI == EPI_WGRAD ? 0 : expert * p.strideB) + n0 + ch * 8);
             }
         }
+        load_b_src(0);
         return true;
     };
 
     // Loads of contraction step `step` into `stage`.  The padding step of an odd step count (the
     // loop works on pairs of steps) re-reads the last valid slice; its A tile is zeroed.
-    const int lda32 = static_cast<int>(p.lda), ldb32 = static_cast<int>(p.ldb);
     // Loads [lo, hi) of the step's list (A loads first, then B loads); lo and hi are constants
     // after unrolling.
     auto issue_part = [&](int step, char *stage, int lo, int hi) {
@@ -366,10 +390,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             } else {
                 int c = c0 + b_crow[i];
                 if (EPI == EPI_WGRAD) c = min(c, c_len - 1);
-                off = static_cast<uint32_t>(b_off[i] + (c_begin + c) * ldb32) * 2u;
+                if (GATHER == GATHER_B)
+                    off = static_cast<uint32_t>(b_off[i] + b_src[GATHER == GATHER_B ? i : 0] * ldb32) * 2u;
+                else
+                    off = static_cast<uint32_t>(b_off[i] + (c_begin + c) * ldb32) * 2u;
             }
             load16_to_lds(((EPI == EPI_SWIGLU && b_up[i]) ? Bup : Bp) + off, sb + i * 1024);
         }
+        if (hi >= A_LOADS + B_LOADS && lo < A_LOADS + B_LOADS) load_b_src(step + 1);   // this step's B loads are out
     };
     constexpr int NL = A_LOADS + B_LOADS;
     auto issue_loads = [&](int step, char *stage) { issue_part(step, stage, 0, NL); };
@@ -738,7 +766,7 @@ template <int BM> struct Waves {
     static constexpr int N = (BM == 256) ? OM_WAVES_N : 2;
 };
 
-template <int BM, int BN, int AKIND, int BKIND, int EPI>
+template <int BM, int BN, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE>
 int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad family
     constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
     if (p.n_experts > MAX_EXPERTS) return OM_ERR_SHAPE;   // the tile table lives in LDS
@@ -746,19 +774,19 @@ int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad f
     const int64_t tiles = static_cast<int64_t>(p.m_tiles_max) * (p.n_cols / BN_OUT);
     if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
     p.total_tiles = static_cast<int>(tiles);
-    ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI>
+    ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI, GATHER>
         <<<dim3(persistent_blocks<BM>(tiles)), dim3(Waves<BM>::M * Waves<BM>::N * 64), 0, st>>>(p);
     return om_launch_status();
 }
 
-template <int AKIND, int BKIND, int EPI>
+template <int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE>
 int launch_rows_auto(GemmParams &p, int64_t rows, hipStream_t st) {
     constexpr int div = (EPI == EPI_SWIGLU) ? 2 : 1;
     const bool big_ok = p.n_cols % (256 / div) == 0;
     const bool few_rows = rows < static_cast<int64_t>(p.n_experts) * 192;
-    if (big_ok && !few_rows) return launch_rows<256, 256, AKIND, BKIND, EPI>(p, rows, st);
+    if (big_ok && !few_rows) return launch_rows<256, 256, AKIND, BKIND, EPI, GATHER>(p, rows, st);
     if (p.n_cols % (128 / div) != 0) return OM_ERR_SHAPE;
-    return launch_rows<128, 128, AKIND, BKIND, EPI>(p, rows, st);
+    return launch_rows<128, 128, AKIND, BKIND, EPI, GATHER>(p, rows, st);
 }
 
 }  // namespace
@@ -801,44 +829,69 @@ extern "C" int om_grouped_gemm_dgrad(const void *output_grad, const void *weight
     return launch_rows_auto<CONTIG, STRIDED, EPI_STORE>(p, rows, om_stream(stream));
 }
 
-extern "C" int om_grouped_gemm_wgrad(const void *output_grad, const void *input, void *weight_grad,
-                                     const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
-                                     int64_t w_stride, void *stream) {
+namespace {
+// weight gradient; `input_rows` != null: contraction row c of `input` is row input_rows[c] of a
+// [src_rows, K] matrix (the token gather folded into the loads)
+int wgrad_launch(const void *output_grad, const void *input, const int32_t *input_rows, int64_t src_rows,
+                 void *weight_grad, const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                 int64_t w_stride, void *stream) {
     if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
     if (!output_grad || !input || !weight_grad || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(output_grad) || !om_aligned16(input) || !om_aligned16(weight_grad)) return OM_ERR_ALIGN;
     GemmParams p = {};
     p.A[0] = static_cast<const uint16_t *>(output_grad);  // [rows, N]: operand rows = n, c = row
-    p.B[0] = static_cast<const uint16_t *>(input);        // [rows, K]
+    p.B[0] = static_cast<const uint16_t *>(input);        // [rows, K] (or [src_rows, K] through input_rows)
     p.C = static_cast<uint16_t *>(weight_grad);           // [G, N, K]
     p.cum = cum_token_counts;
+    p.row_index = input_rows;
     p.lda = N; p.ldb = K; p.ldc = K;
     p.strideC = w_stride ? w_stride : static_cast<int64_t>(N) * K;
-    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideC * G)) return OM_ERR_SHAPE;
+    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideC * G) || !fits31(src_rows * K))
+        return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
     hipStream_t st = om_stream(stream);
-    if (N % 256 == 0 && K % 256 == 0) {
-        p.tiles_e = (N / 256) * (K / 256);
-        const int64_t tiles = static_cast<int64_t>(p.tiles_e) * G;
-        if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
-        p.total_tiles = static_cast<int>(tiles);
-        ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD>
-            <<<dim3(persistent_blocks<256>(tiles)), dim3(Waves<256>::M * Waves<256>::N * 64), 0, st>>>(p);
-    } else {
-        p.tiles_e = (N / 128) * (K / 128);
-        const int64_t tiles = static_cast<int64_t>(p.tiles_e) * G;
-        if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
-        p.total_tiles = static_cast<int>(tiles);
-        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD>
-            <<<dim3(persistent_blocks<128>(tiles)), dim3(256), 0, st>>>(p);
-    }
+    const bool big = N % 256 == 0 && K % 256 == 0;
+    p.tiles_e = big ? (N / 256) * (K / 256) : (N / 128) * (K / 128);
+    const int64_t tiles = static_cast<int64_t>(p.tiles_e) * G;
+    if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
+    p.total_tiles = static_cast<int>(tiles);
+    const dim3 grid_big(persistent_blocks<256>(tiles)), block_big(Waves<256>::M * Waves<256>::N * 64);
+    const dim3 grid_small(persistent_blocks<128>(tiles)), block_small(256);
+    if (big && !input_rows)
+        ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD><<<grid_big, block_big, 0, st>>>(p);
+    else if (big)
+        ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD, GATHER_B><<<grid_big, block_big, 0, st>>>(p);
+    else if (!input_rows)
+        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD><<<grid_small, block_small, 0, st>>>(p);
+    else
+        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD, GATHER_B><<<grid_small, block_small, 0, st>>>(p);
     return om_launch_status();
 }
+}  // namespace
 
-extern "C" int om_merged_mlp_gate_up_fwd(const void *x, const void *w_gate, const void *w_up, void *g,
-                                         void *u, void *h, const int32_t *cum_token_counts,
-                                         int64_t rows, int G, int I, int H, int64_t w_stride,
-                                         void *stream) {
+extern "C" int om_grouped_gemm_wgrad(const void *output_grad, const void *input, void *weight_grad,
+                                     const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                                     int64_t w_stride, void *stream) {
+    return wgrad_launch(output_grad, input, nullptr, 0, weight_grad, cum_token_counts, rows, G, N, K,
+                        w_stride, stream);
+}
+
+extern "C" int om_grouped_gemm_wgrad_gathered(const void *output_grad, const void *input,
+                                              const int32_t *input_rows, int64_t src_rows,
+                                              void *weight_grad, const int32_t *cum_token_counts,
+                                              int64_t rows, int G, int N, int K, int64_t w_stride,
+                                              void *stream) {
+    if (!input_rows) return OM_ERR_NULL;
+    if (src_rows < 1) return OM_ERR_SHAPE;
+    return wgrad_launch(output_grad, input, input_rows, src_rows, weight_grad, cum_token_counts, rows, G,
+                        N, K, w_stride, stream);
+}
+
+namespace {
+// `x_rows` != null: sorted row r of the activations is row x_rows[r] of x [src_rows, H]
+int gate_up_fwd_launch(const void *x, const int32_t *x_rows, int64_t src_rows, const void *w_gate,
+                       const void *w_up, void *g, void *u, void *h, const int32_t *cum_token_counts,
+                       int64_t rows, int G, int I, int H, int64_t w_stride, void *stream) {
     if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 128)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!x || !w_gate || !w_up || !g || !u || !h || !cum_token_counts) return OM_ERR_NULL;
@@ -853,11 +906,34 @@ extern "C" int om_merged_mlp_gate_up_fwd(const void *x, const void *w_gate, cons
     p.C1 = static_cast<uint16_t *>(u);
     p.C2 = static_cast<uint16_t *>(h);
     p.cum = cum_token_counts;
+    p.row_index = x_rows;
     p.lda = H; p.ldb = H; p.ldc = I;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(I) * H;
-    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
+    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G) || !fits31(src_rows * H))
+        return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = I; p.kc = H; p.phases = 1;
+    if (x_rows) return launch_rows_auto<CONTIG, CONTIG, EPI_SWIGLU, GATHER_A>(p, rows, om_stream(stream));
     return launch_rows_auto<CONTIG, CONTIG, EPI_SWIGLU>(p, rows, om_stream(stream));
+}
+}  // namespace
+
+extern "C" int om_merged_mlp_gate_up_fwd(const void *x, const void *w_gate, const void *w_up, void *g,
+                                         void *u, void *h, const int32_t *cum_token_counts,
+                                         int64_t rows, int G, int I, int H, int64_t w_stride,
+                                         void *stream) {
+    return gate_up_fwd_launch(x, nullptr, 0, w_gate, w_up, g, u, h, cum_token_counts, rows, G, I, H,
+                              w_stride, stream);
+}
+
+extern "C" int om_merged_mlp_gate_up_fwd_gathered(const void *x, const int32_t *x_rows, int64_t src_rows,
+                                                  const void *w_gate, const void *w_up, void *g, void *u,
+                                                  void *h, const int32_t *cum_token_counts,
+                                                  int64_t rows, int G, int I, int H, int64_t w_stride,
+                                                  void *stream) {
+    if (rows > 0 && !x_rows) return OM_ERR_NULL;
+    if (src_rows < 1 && rows > 0) return OM_ERR_SHAPE;
+    return gate_up_fwd_launch(x, x_rows, src_rows, w_gate, w_up, g, u, h, cum_token_counts, rows, G, I, H,
+                              w_stride, stream);
 }
 
 extern "C" int om_merged_mlp_down_dgrad(const void *dy, const void *w_down, const void *g, const void *u,

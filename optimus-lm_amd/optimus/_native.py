@@ -81,6 +81,11 @@ SIGNATURES = {
                                       c_int, c_i64, c_void_p]),
     "om_merged_mlp_gate_up_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_void_p, c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
+    "om_merged_mlp_gate_up_fwd_gathered": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p,
+                                                   c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
+                                                   c_int, c_i64, c_void_p]),
+    "om_grouped_gemm_wgrad_gathered": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p,
+                                               c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
     "om_merged_mlp_down_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
     "om_merged_mlp_gate_up_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

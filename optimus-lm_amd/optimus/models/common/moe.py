@@ -303,11 +303,14 @@ class GroupedGemmFunction(torch.autograd.Function):
         return input_grad, merged_weight_grad, None, None, None
 
 
-def _merged_mlp_forward(x, w_gate, w_up, w_down, cum_token_counts):
-    """-> (y, cum, g, u, h).  Fused gate+up+SwiGLU launch, then the down projection."""
+def _merged_mlp_forward(x, w_gate, w_up, w_down, cum_token_counts, x_rows=None):
+    """-> (y, cum, g, u, h).  Fused gate+up+SwiGLU launch, then the down projection.  With
+    `x_rows` (int32 [rows]) the MLP input is x[x_rows] without that matrix being built."""
     _require_bf16(x, w_gate, w_up, w_down)
-    _n.require_cuda_contiguous(x)
+    _n.require_cuda_contiguous(x, x_rows)
     rows, H = x.shape
+    if x_rows is not None:
+        rows = x_rows.shape[0]
     G, I, _ = w_gate.shape
     cum = _device_counts(cum_token_counts, x.device)
     g = torch.empty((rows, I), dtype=x.dtype, device=x.device)
@@ -319,25 +322,32 @@ def _merged_mlp_forward(x, w_gate, w_up, w_down, cum_token_counts):
     if _expert_stride(w_up) != sgu:
         raise _n.NativeLibraryError("gate and up expert weights must share one expert pitch")
     with record_pcl_function("1moeblock--7gmlp_fwd"):
-        _n.check(lib.om_merged_mlp_gate_up_fwd(
-            _n.ptr(x), _n.ptr(w_gate), _n.ptr(w_up), _n.ptr(g), _n.ptr(u), _n.ptr(h), _n.ptr(cum),
-            rows, G, I, H, sgu, _n.stream()), "om_merged_mlp_gate_up_fwd")
+        if x_rows is not None and rows > 0:
+            _n.check(lib.om_merged_mlp_gate_up_fwd_gathered(
+                _n.ptr(x), _n.ptr(x_rows), x.shape[0], _n.ptr(w_gate), _n.ptr(w_up), _n.ptr(g),
+                _n.ptr(u), _n.ptr(h), _n.ptr(cum), rows, G, I, H, sgu, _n.stream()),
+                "om_merged_mlp_gate_up_fwd_gathered")
+        else:
+            _n.check(lib.om_merged_mlp_gate_up_fwd(
+                _n.ptr(x), _n.ptr(w_gate), _n.ptr(w_up), _n.ptr(g), _n.ptr(u), _n.ptr(h), _n.ptr(cum),
+                rows, G, I, H, sgu, _n.stream()), "om_merged_mlp_gate_up_fwd")
         _n.check(lib.om_grouped_gemm_fwd(
             _n.ptr(h), _n.ptr(w_down), _n.ptr(y), _n.ptr(cum), rows, G, H, I,
             _expert_stride(w_down), _n.stream()), "om_grouped_gemm_fwd")
     return y, cum, g, u, h
 
 
-def _merged_mlp_backward(dy, x, w_gate, w_up, w_down, cum, g, u, h):
-    """-> (dx, dw_gate [G,I,H], dw_up [G,I,H], dw_down [G,H,I]), all freshly allocated."""
+def _merged_mlp_backward(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows=None):
+    """-> (dx, dw_gate [G,I,H], dw_up [G,I,H], dw_down [G,H,I]), all freshly allocated.  With
+    `x_rows` the MLP input was x[x_rows]; dx is then the gradient of that gathered matrix."""
     dy = dy.contiguous()
-    rows, H = x.shape
+    rows, H = dy.shape
     G, I, _ = w_gate.shape
     lib = _n.lib()
     st = _n.stream()
     dg = torch.empty_like(g)
     du = torch.empty_like(u)
-    dx = torch.empty_like(x)
+    dx = torch.empty((rows, H), dtype=x.dtype, device=x.device)
     dw_gate = torch.empty((G, I, H), dtype=x.dtype, device=x.device)
     dw_up = torch.empty((G, I, H), dtype=x.dtype, device=x.device)
     dw_down = torch.empty((G, H, I), dtype=x.dtype, device=x.device)
@@ -347,10 +357,16 @@ def _merged_mlp_backward(dy, x, w_gate, w_up, w_down, cum, g, u, h):
         _n.check(lib.om_merged_mlp_down_dgrad(_n.ptr(dy), _n.ptr(w_down), _n.ptr(g), _n.ptr(u),
                                               _n.ptr(dg), _n.ptr(du), _n.ptr(cum), rows, G, I, H,
                                               _expert_stride(w_down), st), "om_merged_mlp_down_dgrad")
-        _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(dg), _n.ptr(x), _n.ptr(dw_gate), _n.ptr(cum),
-                                           rows, G, I, H, 0, st), "om_grouped_gemm_wgrad(gate)")
-        _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(du), _n.ptr(x), _n.ptr(dw_up), _n.ptr(cum),
-                                           rows, G, I, H, 0, st), "om_grouped_gemm_wgrad(up)")
+        if x_rows is not None and rows > 0:
+            for grad, dw, name in ((dg, dw_gate, "gate"), (du, dw_up, "up")):
+                _n.check(lib.om_grouped_gemm_wgrad_gathered(
+                    _n.ptr(grad), _n.ptr(x), _n.ptr(x_rows), x.shape[0], _n.ptr(dw), _n.ptr(cum), rows,
+                    G, I, H, 0, st), f"om_grouped_gemm_wgrad_gathered({name})")
+        else:
+            _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(dg), _n.ptr(x), _n.ptr(dw_gate), _n.ptr(cum),
+                                               rows, G, I, H, 0, st), "om_grouped_gemm_wgrad(gate)")
+            _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(du), _n.ptr(x), _n.ptr(dw_up), _n.ptr(cum),
+                                               rows, G, I, H, 0, st), "om_grouped_gemm_wgrad(up)")
         _n.check(lib.om_merged_mlp_gate_up_dgrad(_n.ptr(dg), _n.ptr(du), _n.ptr(w_gate),
                                                  _n.ptr(w_up), _n.ptr(dx), _n.ptr(cum), rows, G,
                                                  I, H, _expert_stride(w_gate), st),
@@ -379,6 +395,36 @@ class MergedMLPFunction(torch.autograd.Function):
         return dx, dw_gate, dw_up, dw_down, None
 
 
+class GatheredMergedMLPFunction(torch.autograd.Function):
+    """PrepareInputForGroupGemmFunction followed by MergedMLPFunction (reference moe.py:217-282 and
+    :396-405) without the gathered copy of the activations: the gate/up forward GEMM and the two
+    gate/up weight-gradient GEMMs read hidden_states through input_indices.  Bit-identical to the
+    two functions in sequence; backward ends with the same per-token reduction of the routed rows'
+    gradients (shuffle_sub_matrix_reduce)."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, input_indices, cum_expert_counts_ep, output_indices, w_gate, w_up,
+                w_down, cum_token_counts):
+        hidden_states = hidden_states.contiguous()
+        y, cum, g, u, h = _merged_mlp_forward(hidden_states, w_gate, w_up, w_down, cum_token_counts,
+                                              x_rows=input_indices)
+        ctx.save_for_backward(hidden_states, input_indices, cum_expert_counts_ep, output_indices, w_gate,
+                              w_up, w_down, cum, g, u, h)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        (hidden_states, input_indices, cum_expert_counts_ep, output_indices, w_gate, w_up, w_down, cum,
+         g, u, h) = ctx.saved_tensors
+        dx_rows, dw_gate, dw_up, dw_down = _merged_mlp_backward(dy, hidden_states, w_gate, w_up, w_down,
+                                                                cum, g, u, h, x_rows=input_indices)
+        with record_pcl_function("1moeblock--6gmlp_input_prep_bwd"):
+            hidden_states_grad = torch.empty_like(hidden_states)
+            pcl_xpu_customops.shuffle_sub_matrix_reduce(dx_rows, cum_expert_counts_ep, output_indices,
+                                                        hidden_states_grad)
+        return hidden_states_grad, None, None, None, dw_gate, dw_up, dw_down, None
+
+
 class GroupMLPFunction(torch.autograd.Function):
     """Un-merged layout of the reference (moe.py:43-161): weights arrive as 3*N separate
     [out, in] tensors (gate_0, up_0, down_0, gate_1, ...).  They must sit at one constant pitch
@@ -401,6 +447,39 @@ class GroupMLPFunction(torch.autograd.Function):
         for n in range(dwg.shape[0]):
             flat += [dwg[n], dwu[n], dwd[n]]
         return (dx, None, None, *flat)
+
+
+class GatheredGroupMLPFunction(torch.autograd.Function):
+    """GroupMLPFunction on hidden_states[input_indices] without the gathered copy (see
+    GatheredMergedMLPFunction); weights as in GroupMLPFunction."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, input_indices, cum_expert_counts_ep, output_indices, cum_token_counts,
+                *weight_tuple):
+        N = len(weight_tuple) // 3
+        wg, wu, wd = [_strided_expert_view([weight_tuple[3 * n + j] for n in range(N)])
+                      for j in range(3)]
+        hidden_states = hidden_states.contiguous()
+        y, cum, g, u, h = _merged_mlp_forward(hidden_states, wg, wu, wd, cum_token_counts,
+                                              x_rows=input_indices)
+        ctx.save_for_backward(hidden_states, input_indices, cum_expert_counts_ep, output_indices, wg, wu,
+                              wd, cum, g, u, h)
+        return y
+
+    @staticmethod
+    def backward(ctx, output_grad):
+        (hidden_states, input_indices, cum_expert_counts_ep, output_indices, wg, wu, wd, cum, g, u,
+         h) = ctx.saved_tensors
+        dx_rows, dwg, dwu, dwd = _merged_mlp_backward(output_grad, hidden_states, wg, wu, wd, cum, g, u, h,
+                                                      x_rows=input_indices)
+        with record_pcl_function("1moeblock--6gmlp_input_prep_bwd"):
+            hidden_states_grad = torch.empty_like(hidden_states)
+            pcl_xpu_customops.shuffle_sub_matrix_reduce(dx_rows, cum_expert_counts_ep, output_indices,
+                                                        hidden_states_grad)
+        flat = []
+        for n in range(dwg.shape[0]):
+            flat += [dwg[n], dwu[n], dwd[n]]
+        return (hidden_states_grad, None, None, None, None, *flat)
 
 
 def _strided_expert_view(weights):
@@ -538,11 +617,22 @@ class MergedMLP(nn.Module):
         return MergedMLPFunction.apply(input, self.gate_proj_merged_weight, self.up_proj_merged_weight,
                                        self.down_proj_merged_weight, cum_token_counts)
 
+    def forward_gathered(self, hidden_states, input_indices, cum_expert_counts_ep, output_indices,
+                         cum_token_counts):
+        """forward(hidden_states[input_indices], cum_token_counts) with the gather folded into the
+        GEMMs; the two index arrays after input_indices serve the backward's per-token reduction."""
+        return GatheredMergedMLPFunction.apply(hidden_states, input_indices, cum_expert_counts_ep,
+                                               output_indices, self.gate_proj_merged_weight,
+                                               self.up_proj_merged_weight, self.down_proj_merged_weight,
+                                               cum_token_counts)
+
 
 def expert_computation(hidden_states, routing_weights, selected_experts, expert_start_idx,
-                       expert_end_idx, experts_fn, num_total_experts):
+                       expert_end_idx, experts_fn, num_total_experts, gathered_experts_fn=None):
     """K1..K6 for 2-D hidden_states [T,H]: permute, run `experts_fn(ggemm_input, cum_token_counts)`,
-    combine.  Shared by the OLMoE and DeepSeek-V3 blocks."""
+    combine.  Shared by the OLMoE and DeepSeek-V3 blocks.  With `gathered_experts_fn(hidden_states,
+    input_indices, cum_expert_counts_ep, output_indices, cum_token_counts)` the experts read the
+    tokens through the index and K4's gathered copy is not built."""
     T, K = selected_experts.shape
     with record_pcl_function("1moeblock--3index_calculation"):
         (cum_token_counts, cum_expert_counts_ep, input_indices, output_indices,
@@ -555,9 +645,13 @@ def expert_computation(hidden_states, routing_weights, selected_experts, expert_
     input_indices = input_indices[:num_routed_tokens]
     output_indices = output_indices[:num_routed_tokens]
     selected_experts_indices = selected_experts_indices[:num_routed_tokens]
-    ggemm_input = PrepareInputForGroupGemmFunction.apply(hidden_states, input_indices,
-                                                         cum_expert_counts_ep, output_indices)
-    ggemm_output = experts_fn(ggemm_input, cum_token_counts)
+    if gathered_experts_fn is not None:
+        ggemm_output = gathered_experts_fn(hidden_states, input_indices, cum_expert_counts_ep,
+                                           output_indices, cum_token_counts)
+    else:
+        ggemm_input = PrepareInputForGroupGemmFunction.apply(hidden_states, input_indices,
+                                                             cum_expert_counts_ep, output_indices)
+        ggemm_output = experts_fn(ggemm_input, cum_token_counts)
     return GroupGemmOutputReductionFunction.apply(ggemm_output, routing_weights, cum_expert_counts_ep,
                                                   selected_experts_indices, input_indices,
                                                   output_indices)
@@ -598,6 +692,8 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
                                       "(moe.py:459-464) and is not part of this build")
         # fp32 router logits (x.float() @ Wg.float().T) instead of model-dtype logits
         self.router_logits_fp32 = bool(getattr(config, "router_logits_fp32", False))
+        # merged experts read the tokens through input_indices instead of a gathered copy
+        self.fuse_input_gather = bool(getattr(config, "fuse_input_gather", True))
 
     def _experts_fn(self, ggemm_input, cum_token_counts):
         if isinstance(self.experts, MergedMLP):
@@ -607,6 +703,18 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
         for expert in self.experts:
             mlp_params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
         return GroupMLPFunction.apply(ggemm_input, cum_token_counts, False, *mlp_params)
+
+    def _gathered_experts_fn(self, hidden_states, input_indices, cum_expert_counts_ep, output_indices,
+                             cum_token_counts):
+        if isinstance(self.experts, MergedMLP):
+            return self.experts.forward_gathered(hidden_states, input_indices, cum_expert_counts_ep,
+                                                 output_indices, cum_token_counts)
+        pack_expert_weights(self.experts)
+        mlp_params = []
+        for expert in self.experts:
+            mlp_params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
+        return GatheredGroupMLPFunction.apply(hidden_states, input_indices, cum_expert_counts_ep,
+                                              output_indices, cum_token_counts, *mlp_params)
 
     def forward(self, hidden_states):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
@@ -626,9 +734,10 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
 
         def expert_computation_block(hidden_states, selected_experts, routing_weights):
             b, s, h = hidden_states.shape
+            gathered = self._gathered_experts_fn if self.fuse_input_gather else None
             out = expert_computation(hidden_states.reshape(-1, h), routing_weights, selected_experts,
                                      self.expert_start_idx, self.expert_end_idx, self._experts_fn,
-                                     self.num_experts)
+                                     self.num_experts, gathered_experts_fn=gathered)
             return out.reshape(b, s, h)
 
         args = [hidden_states, selected_experts, routing_weights]

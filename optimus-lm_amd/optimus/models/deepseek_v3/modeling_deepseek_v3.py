@@ -140,12 +140,23 @@ class DeepseekV3ParallelMoE(nn.Module):
             params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
         return _moe.GroupMLPFunction.apply(ggemm_input, cum_token_counts, False, *params)
 
+    def _gathered_experts_fn(self, hidden_states, input_indices, cum_expert_counts_ep, output_indices,
+                             cum_token_counts):
+        _moe.pack_expert_weights(self.experts)
+        params = []
+        for expert in self.experts:
+            params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
+        return _moe.GatheredGroupMLPFunction.apply(hidden_states, input_indices, cum_expert_counts_ep,
+                                                   output_indices, cum_token_counts, *params)
+
     def moe(self, hidden_states, topk_indices, topk_weights):
         """Routed part for [T,H] hidden_states (reference :221-244): fp32 weights, fp32 sum over a
-        token's local experts, one rounding to the activation dtype."""
+        token's local experts, one rounding to the activation dtype.  The local experts read their
+        tokens through the permutation index (no gathered copy of the activations)."""
+        gathered = self._gathered_experts_fn if getattr(self.config, "fuse_input_gather", True) else None
         return _moe.expert_computation(hidden_states, topk_weights, topk_indices,
                                        self.expert_start_idx, self.expert_end_idx, self._experts_fn,
-                                       self.config.n_routed_experts)
+                                       self.config.n_routed_experts, gathered_experts_fn=gathered)
 
     def forward(self, hidden_states):
         topk_indices, topk_weights = self.gate(hidden_states)

@@ -107,3 +107,44 @@ def test_merged_mlp_fused(cuda, kind, G, rows, I, H):
     assert max_abs(y.float().cpu(), yr.detach()) <= 2e-2 * max(1.0, float(yr.abs().max()))
     for name, a, b in zip(("dx", "dwg", "dwu", "dwd"), dev, ref):
         assert mean_rel(a.grad.float().cpu(), b.grad) <= 1e-2, name
+
+
+@pytest.mark.parametrize("T,K,N,start,end,I,H,skew", [
+    (4096, 8, 64, 0, 64, 512, 512, 0.0),      # 256x256 tiles, forward and weight gradient
+    (512, 2, 8, 0, 8, 128, 384, 0.0),         # 128x128 tiles
+    (3000, 4, 16, 4, 12, 256, 256, 1.5),      # expert window: only part of the pairs is routed; skew
+    (70, 8, 64, 0, 64, 128, 128, 3.0),        # most experts empty, a few rows each
+    (16384, 8, 64, 0, 64, 1024, 2048, 0.0),   # C3
+])
+def test_gathered_merged_mlp_is_bit_identical(cuda, T, K, N, start, end, I, H, skew):
+    """The token gather folded into the GEMM loads (om_merged_mlp_gate_up_fwd_gathered,
+    om_grouped_gemm_wgrad_gathered) against gather-then-GEMM (om_index_gather + the plain entry
+    points): the same products are summed in the same order, so outputs and every gradient must be
+    equal bit for bit."""
+    from optimus.models.common.moe import (GatheredMergedMLPFunction, MergedMLPFunction,
+                                           PrepareInputForGroupGemmFunction, build_token_permutation)
+    from util import routed_experts
+    G = end - start
+    g = torch.Generator().manual_seed(T + I)
+    se = routed_experts(T, N, K, seed=T + K, skew=skew).to(cuda)
+    cum, cum_ep, ii, oi, _ = build_token_permutation(se, start, end)
+    rows = int(cum[-1].item())
+    ii, oi = ii[:rows], oi[:rows]
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ws = [(torch.randn(G, I, H, generator=g) * 0.05).to(torch.bfloat16),
+          (torch.randn(G, I, H, generator=g) * 0.05).to(torch.bfloat16),
+          (torch.randn(G, H, I, generator=g) * 0.05).to(torch.bfloat16)]
+    dy = torch.randn(rows, H, generator=g).to(torch.bfloat16).to(cuda)
+    results = []
+    for gathered in (False, True):
+        xd = x.to(cuda).requires_grad_(True)
+        wd = [w.to(cuda).requires_grad_(True) for w in ws]
+        if gathered:
+            y = GatheredMergedMLPFunction.apply(xd, ii, cum_ep, oi, *wd, cum)
+        else:
+            y = MergedMLPFunction.apply(PrepareInputForGroupGemmFunction.apply(xd, ii, cum_ep, oi), *wd, cum)
+        y.backward(dy)
+        results.append([y.detach(), xd.grad] + [w.grad for w in wd])
+    for name, a, b in zip(("y", "dx", "dw_gate", "dw_up", "dw_down"), *results):
+        assert torch.equal(a, b), name
+    assert results[0][0].shape == (rows, H) and bool(torch.isfinite(results[1][0].float()).all())

@@ -165,6 +165,27 @@ def test_activation_checkpointing_recomputes_identically(cuda):
         assert torch.equal(x0, x1)
 
 
+@pytest.mark.parametrize("name,merged", [("C4", True), ("C1", False)])
+def test_gather_fusion_switch_changes_no_bit(cuda, name, merged):
+    """The experts read their tokens through input_indices by default; with the switch off the block
+    builds ggemm_input = hidden_states[input_indices] first (the reference's K4).  Same products, same
+    order of summation: output and every gradient are equal bit for bit."""
+    inp = sc.moe_inputs(name)
+    c = inp["cfg"]
+    res = []
+    for fuse in (True, False):
+        blk = _olmoe_block(inp, cuda, merged=merged)
+        assert blk.fuse_input_gather is True
+        blk.fuse_input_gather = fuse
+        xi = inp["x"].to(cuda).view(1, c["T"], c["H"]).requires_grad_(True)
+        o, _ = blk(xi)
+        o.backward(inp["dout"].to(cuda).view_as(o))
+        res.append([o, xi.grad] + [p.grad for p in blk.parameters()])
+    assert len(res[0]) == len(res[1]) >= 5
+    for x0, x1 in zip(*res):
+        assert torch.equal(x0, x1)
+
+
 @pytest.mark.parametrize("ep_ind", [0, 3])
 def test_dsv3_block_one_rank_share(cuda, ep_ind):
     """C5 at reduced size: DeepseekV3ParallelMoE with expert_parallelism=8 (32 of 256 routed experts
