@@ -119,6 +119,15 @@ def test_grouped_gemms(lib):
     assert lib.om_merged_mlp_gate_up_fwd(P, P, None, P, P, P, P, 131072, 64, 1024, 2048, 0, None) == NULL
     assert lib.om_merged_mlp_down_dgrad(P, P, P, P, P, ODD, P, 131072, 64, 1024, 2048, 0, None) == ALIGN
     assert lib.om_merged_mlp_gate_up_dgrad(P, P, P, P, None, P, 131072, 64, 1024, 2048, 0, None) == NULL
+    # the forms that read the tokens through an index
+    g = (131072, 64, 1024, 2048, 0, None)
+    assert lib.om_merged_mlp_gate_up_fwd_gathered(P, None, 16384, P, P, P, P, P, P, *g) == NULL      # no index
+    assert lib.om_merged_mlp_gate_up_fwd_gathered(P, P, 0, P, P, P, P, P, P, *g) == SHAPE            # no source rows
+    assert lib.om_merged_mlp_gate_up_fwd_gathered(P, P, 1 << 21, P, P, P, P, P, P, *g) == SHAPE      # source > 2^31 elements
+    assert lib.om_merged_mlp_gate_up_fwd_gathered(P, None, 0, P, P, P, P, P, P, 0, 64, 1024, 2048, 0, None) == OK
+    assert lib.om_grouped_gemm_wgrad_gathered(P, P, None, 16384, P, P, *g) == NULL
+    assert lib.om_grouped_gemm_wgrad_gathered(P, P, P, 0, P, P, *g) == SHAPE
+    assert lib.om_grouped_gemm_wgrad_gathered(P, P, P, 16384, ODD, P, *g) == ALIGN
 
 
 def test_check_raises_with_the_library_text():
