@@ -18,12 +18,13 @@ def from_bits(a, dtype):
 
 
 def max_abs(a, b):
-    return float((a.double() - b.double()).abs().max())
+    return float((a.detach().double() - b.detach().double()).abs().max())
 
 
 def mean_rel(a, b):
     """mean(|a-b|) / mean(|b|) — the layer-parity figure of merit."""
-    return float((a.double() - b.double()).abs().mean() / b.double().abs().mean().clamp_min(1e-30))
+    a, b = a.detach().double(), b.detach().double()
+    return float((a - b).abs().mean() / b.abs().mean().clamp_min(1e-30))
 
 
 def routed_experts(T, N, K, seed, skew=0.0):
