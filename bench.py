@@ -11,7 +11,7 @@ Secondary workload (the `adamw` object of the same JSON line): the flat-buffer m
 AdamW step over 6.9e9 parameters (BASELINE config C2).
 
 Kernel durations come from HIP events recorded on the launch stream around the C-ABI calls.  An
-untimed survey pass brackets every call (the `kernels` table, the all-GEMM aggregate, and which
+untimed profiling pass brackets every call (the `kernels` table, the all-GEMM aggregate, and which
 entry point is dominant); inside the timed steps only the dominant entry point's launches are
 bracketed, because every event pair leaves a gap of about 10 us on the stream, and the roofline
 figure is taken from those.  The CPU baselines time the oracle's PyTorch-CPU restatements of the
@@ -106,15 +106,15 @@ def bench_moe(args, device):
 
     for _ in range(args.warmup):
         step()
-    # Survey pass (not the metric): every entry point bracketed by events, which gives the per-kernel
+    # Profiling pass (not the metric): every entry point bracketed by events, which gives the per-kernel
     # table and names the dominant kernel.  An event pair costs a gap of about 10 us on the stream,
     # so the timed steps below bracket the dominant entry point only.
     _, per = run(max(3, min(args.steps, 10)))
-    n_survey = max(3, min(args.steps, 10))
+    n_profiled = max(3, min(args.steps, 10))
     TR = T * K
     prod_flops = 2.0 * TR * H * I
-    gemm_ms = sum(sum(v) for k, v in per.items() if k in GEMM_ENTRY_PRODUCTS) / n_survey
-    kernels = {k: {"launches_per_step": len(v) / n_survey, "avg_ms": sum(v) / len(v)}
+    gemm_ms = sum(sum(v) for k, v in per.items() if k in GEMM_ENTRY_PRODUCTS) / n_profiled
+    kernels = {k: {"launches_per_step": len(v) / n_profiled, "avg_ms": sum(v) / len(v)}
                for k, v in sorted(per.items())}
     # dominant kernel = the entry point with the largest summed duration
     dom = max((k for k in per if k in GEMM_ENTRY_PRODUCTS), key=lambda k: sum(per[k]))
@@ -125,7 +125,7 @@ def bench_moe(args, device):
     roofline = {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1),
                 "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
-                "all_expert_gemms": {"from": "survey pass with every entry point bracketed by events",
+                "all_expert_gemms": {"from": "untimed profiling pass with every entry point bracketed by events",
                                      "flops_per_step": 9 * prod_flops, "ms_per_step": round(gemm_ms, 3),
                                      "achieved": round(9 * prod_flops / (gemm_ms * 1e-3) / 1e12, 1),
                                      "frac": round(9 * prod_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}}
