@@ -177,6 +177,9 @@ class GateSoftmaxTopkFunction(torch.autograd.Function):
         ctx.save_for_backward(x, weight, logits, experts)
         ctx.norm_topk_prob = bool(norm_topk_prob)
         ctx.mark_non_differentiable(experts)
+        # an output nobody differentiates (the logits without an auxiliary loss) arrives as None in
+        # backward instead of a tensor of zeros that would have to be filled and added
+        ctx.set_materialize_grads(False)
         return weights, experts, logits
 
     @staticmethod
@@ -184,14 +187,19 @@ class GateSoftmaxTopkFunction(torch.autograd.Function):
         x, weight, logits, experts = ctx.saved_tensors
         T, N = logits.shape
         K = experts.shape[1]
-        weights_grad = weights_grad.contiguous()
-        dlogits = torch.empty_like(logits)
-        _n.check(_n.lib().om_route_softmax_topk_bwd(
-            _n.ptr(logits), _n.OM_F32, _n.ptr(experts), _n.ptr(weights_grad),
-            _n.dtype_code(weights_grad), T, N, K, int(ctx.norm_topk_prob), _n.ptr(dlogits),
-            _n.stream()), "om_route_softmax_topk_bwd")
-        if logits_grad is not None:
-            dlogits = dlogits + logits_grad
+        if weights_grad is None and logits_grad is None:
+            return None, None, None, None, None
+        if weights_grad is None:
+            dlogits = logits_grad.to(torch.float32).contiguous()
+        else:
+            weights_grad = weights_grad.contiguous()
+            dlogits = torch.empty_like(logits)
+            _n.check(_n.lib().om_route_softmax_topk_bwd(
+                _n.ptr(logits), _n.OM_F32, _n.ptr(experts), _n.ptr(weights_grad),
+                _n.dtype_code(weights_grad), T, N, K, int(ctx.norm_topk_prob), _n.ptr(dlogits),
+                _n.stream()), "om_route_softmax_topk_bwd")
+            if logits_grad is not None:
+                dlogits = dlogits + logits_grad
         dx, dw = _gate_backward(x, weight, dlogits, ctx.needs_input_grad)
         return dx, dw, None, None, None
 
@@ -587,7 +595,12 @@ class GroupGemmOutputReductionFunction(torch.autograd.Function):
          output_indices) = ctx.saved_tensors
         final_hidden_states_grad = final_hidden_states_grad.contiguous()
         ggemm_output_grad = torch.empty_like(ggemm_output)
-        routing_weights_grad = torch.zeros_like(routing_weights)
+        # the kernel writes the entry of every routed (token, k) pair; pairs outside the expert
+        # window stay zero (the reference pre-zeroes the whole tensor, moe.py:336)
+        if output_indices.shape[0] == routing_weights.numel():
+            routing_weights_grad = torch.empty_like(routing_weights)
+        else:
+            routing_weights_grad = torch.zeros_like(routing_weights)
         with record_pcl_function("1moeblock--8gmlp_output_reduction_bwd"):
             pcl_xpu_customops.reduce_ggemm_output_backward(
                 final_hidden_states_grad, ggemm_output, routing_weights, cum_expert_counts_ep,
