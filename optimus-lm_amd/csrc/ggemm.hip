@@ -836,7 +836,9 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inpu
                  void *weight_grad, const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                  int64_t w_stride, void *stream) {
     if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
-    if (!output_grad || !input || !weight_grad || !cum_token_counts) return OM_ERR_NULL;
+    // rows == 0 (nothing routed to these experts): the activations may be empty tensors without
+    // storage; the launch then only writes zeros
+    if (!weight_grad || !cum_token_counts || (rows > 0 && (!output_grad || !input))) return OM_ERR_NULL;
     if (!om_aligned16(output_grad) || !om_aligned16(input) || !om_aligned16(weight_grad)) return OM_ERR_ALIGN;
     GemmParams p = {};
     p.A[0] = static_cast<const uint16_t *>(output_grad);  // [rows, N]: operand rows = n, c = row

@@ -148,3 +148,24 @@ def test_gathered_merged_mlp_is_bit_identical(cuda, T, K, N, start, end, I, H, s
     for name, a, b in zip(("y", "dx", "dw_gate", "dw_up", "dw_down"), *results):
         assert torch.equal(a, b), name
     assert results[0][0].shape == (rows, H) and bool(torch.isfinite(results[1][0].float()).all())
+
+
+def test_gathered_merged_mlp_with_no_routed_rows(cuda):
+    """An expert window that receives no token: empty output, zero weight gradients, zero input
+    gradient, no launch on empty index arrays."""
+    from optimus.models.common.moe import GatheredMergedMLPFunction, build_token_permutation
+    T, K, H, I, G = 64, 2, 128, 128, 2
+    se = torch.zeros(T, K, dtype=torch.int64, device=cuda)
+    se[:, 1] = 1                                     # every token picks experts 0 and 1
+    cum, cum_ep, ii, oi, _ = build_token_permutation(se, 4, 6)   # window [4, 6): nothing routed
+    assert int(cum[-1].item()) == 0
+    x = torch.randn(T, H, device=cuda).to(torch.bfloat16).requires_grad_(True)
+    ws = [torch.randn(G, I, H, device=cuda).to(torch.bfloat16).requires_grad_(True),
+          torch.randn(G, I, H, device=cuda).to(torch.bfloat16).requires_grad_(True),
+          torch.randn(G, H, I, device=cuda).to(torch.bfloat16).requires_grad_(True)]
+    y = GatheredMergedMLPFunction.apply(x, ii[:0], cum_ep, oi[:0], *ws, cum)
+    assert y.shape == (0, H)
+    y.sum().backward()
+    assert float(x.grad.abs().max()) == 0.0
+    for w in ws:
+        assert float(w.grad.abs().max()) == 0.0

@@ -186,6 +186,39 @@ def test_gather_fusion_switch_changes_no_bit(cuda, name, merged):
         assert torch.equal(x0, x1)
 
 
+@pytest.mark.parametrize("merged", [True, False])
+def test_block_whose_expert_window_gets_no_token(cuda, merged):
+    """An expert-parallel rank none of whose experts is chosen by any token: the block must run
+    forward and backward on empty routed arrays, give zero output, zero input gradient from the
+    experts and zero expert-weight gradients (the gate still gets its gradient through nothing)."""
+    from optimus.mapper import ParallelDpPpEpTpMapper
+    from optimus.models.common.moe import FastOlmoeParallelSparseMoeBlock
+    from optimus.models.olmoe.configuration_olmoe import OlmoeParallelConfig
+    T, H, I, N, K = 256, 256, 128, 8, 2
+    cfg = OlmoeParallelConfig(hidden_size=H, intermediate_size=I, num_experts=N, num_experts_per_tok=K,
+                              norm_topk_prob=True, use_fast_moe=True, use_merged_mlp_in_fast_moe=merged,
+                              expert_parallelism=4)
+    cfg.router_logits_fp32 = True
+    blk = FastOlmoeParallelSparseMoeBlock(cfg, ParallelDpPpEpTpMapper(expert_parallelism=4, rank=3))
+    blk = blk.to(cuda).to(torch.bfloat16)
+    assert (blk.expert_start_idx, blk.expert_end_idx) == (6, 8)
+    g = torch.Generator().manual_seed(3)
+    x = (torch.rand(1, T, H, generator=g) + 0.5).to(torch.bfloat16).to(cuda).requires_grad_(True)   # positive
+    with torch.no_grad():
+        w = torch.full((N, H), -1.0)
+        w[0] = 1.0
+        w[1] = 0.5                       # every token ranks experts 0 and 1 first
+        blk.gate.weight.copy_(w)
+        for p in blk.experts.parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * 0.05)
+    out, _ = blk(x)
+    assert out.shape == x.shape and float(out.detach().abs().max()) == 0.0
+    out.backward(torch.ones_like(out))
+    assert float(x.grad.abs().max()) == 0.0
+    for p in blk.experts.parameters():
+        assert p.grad is not None and float(p.grad.abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("ep_ind", [0, 3])
 def test_dsv3_block_one_rank_share(cuda, ep_ind):
     """C5 at reduced size: DeepseekV3ParallelMoE with expert_parallelism=8 (32 of 256 routed experts
