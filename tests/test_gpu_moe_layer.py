@@ -82,6 +82,45 @@ def test_fast_block_fwd_bwd(cuda, name, scale):
         assert max_abs(a, gref) <= MAX_ABS * max(1.0, float(gref.abs().max())), (k, max_abs(a, gref))
 
 
+@pytest.mark.parametrize("T,H,I,N,K,renorm", [
+    (1, 128, 128, 4, 1, False),        # one token, one expert per token
+    (3, 512, 128, 8, 2, True),
+    (33, 384, 256, 8, 8, False),       # every expert for every token; H not a multiple of 512
+    (257, 512, 128, 64, 8, True),      # about 32 rows per expert, a partial last 64-token stage
+    (100, 512, 256, 130, 5, False),    # expert count that is no multiple of 32 or 64
+    (640, 256, 384, 6, 3, True),       # ffn size a multiple of 128 but not of 256
+])
+def test_fast_block_odd_small_shapes(cuda, T, H, I, N, K, renorm):
+    """Whole block, forward and backward, on sizes that exercise the edges of the tilings (single
+    rows, partial tiles and stages, experts without rows, the small tile shape) against the fp32
+    restatement of the reference block."""
+    g = torch.Generator().manual_seed(1000 * T + N)
+    bf = lambda t: t.to(torch.bfloat16)
+    inp = {"cfg": {"T": T, "H": H, "I": I, "N": N, "K": K, "norm_topk_prob": renorm}, "logits": None,
+           "x": bf(torch.randn(T, H, generator=g)), "gate_w": bf(torch.randn(N, H, generator=g) * 0.1),
+           "w_gate": bf(torch.randn(N, I, H, generator=g) * 0.05), "w_up": bf(torch.randn(N, I, H, generator=g) * 0.05),
+           "w_down": bf(torch.randn(N, H, I, generator=g) * 0.05), "dout": bf(torch.randn(T, H, generator=g))}
+    ref_out, ref_logits, ref_grads = _reference(inp)
+    if R.min_topk_gap_ulps(torch.softmax(ref_logits, 1), K) <= 4.0:
+        pytest.skip("near-tie in the routing scores of this seed")
+    blk = _olmoe_block(inp, cuda)
+    x = inp["x"].to(cuda).view(1, T, H).requires_grad_(True)
+    out, logits = blk(x)
+    out.backward(inp["dout"].to(cuda).view_as(out))
+    _, e_ref, _ = R.olmoe_router(ref_logits, K, renorm, torch.float32)
+    _, e_gpu, _ = R.olmoe_router(logits.float().cpu(), K, renorm, torch.float32)
+    assert torch.equal(e_ref, e_gpu)
+    o = out.detach().float().cpu().view(T, H)
+    assert max_abs(o, ref_out) <= MAX_ABS * max(1.0, float(ref_out.abs().max())) and mean_rel(o, ref_out) <= 6e-3
+    got = {"x": x.grad.view(T, H), "gate_w": blk.gate.weight.grad,
+           "w_gate": blk.experts.gate_proj_merged_weight.grad, "w_up": blk.experts.up_proj_merged_weight.grad,
+           "w_down": blk.experts.down_proj_merged_weight.grad}
+    for k, gref in ref_grads.items():
+        a = got[k].float().cpu()
+        assert mean_rel(a, gref) <= 1.5e-2, (k, mean_rel(a, gref))
+        assert max_abs(a, gref) <= MAX_ABS * max(1.0, float(gref.abs().max())), (k, max_abs(a, gref))
+
+
 def test_fast_block_injected_logits_skewed(cuda):
     """C4: Zipf-skewed routing injected at the functional level (router logits given): many experts
     get 0-8 rows, a few get hundreds.  Expert computation only (router excluded), fwd+bwd."""
