@@ -301,6 +301,20 @@ int om_grouped_gemm_wgrad(const void *output_grad, const void *input, void *weig
                           const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                           int64_t w_stride, void *stream);
 
+/* The same three products for float32 modules (GroupedGemmFunction runs in the module's dtype,
+ * moe.py:174-178, :201-210; the reference's small CPU-runnable configuration is float32): fp32
+ * operands, fp32 MFMA accumulation, fp32 results.  N and K multiples of 64, w_stride a multiple
+ * of 4.  Built for parity at fp32 accuracy, not tuned.                                       */
+int om_grouped_gemm_fwd_f32(const float *input, const float *weight, float *output,
+                            const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                            int64_t w_stride, void *stream);
+int om_grouped_gemm_dgrad_f32(const float *output_grad, const float *weight, float *input_grad,
+                              const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                              int64_t w_stride, void *stream);
+int om_grouped_gemm_wgrad_f32(const float *output_grad, const float *input, float *weight_grad,
+                              const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                              int64_t w_stride, void *stream);
+
 /* Merged-MLP fusions, replacing the three GroupedGemmFunction calls and the two torch
  * elementwise ops of MergedMLP.forward (moe.py:396-405) and their autograd backward:
  *   om_merged_mlp_gate_up_fwd : g = x@Wg[e].T, u = x@Wu[e].T, h = silu(g)*u in one kernel

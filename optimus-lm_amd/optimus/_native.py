@@ -79,6 +79,12 @@ SIGNATURES = {
                                       c_int, c_i64, c_void_p]),
     "om_grouped_gemm_wgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
                                       c_int, c_i64, c_void_p]),
+    "om_grouped_gemm_fwd_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
+                                        c_int, c_i64, c_void_p]),
+    "om_grouped_gemm_dgrad_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
+                                          c_int, c_i64, c_void_p]),
+    "om_grouped_gemm_wgrad_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
+                                          c_int, c_i64, c_void_p]),
     "om_merged_mlp_gate_up_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_void_p, c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
     "om_merged_mlp_gate_up_fwd_gathered": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p,

@@ -48,8 +48,25 @@ def _expert_stride(weight):
 def _require_bf16(*tensors):
     for t in tensors:
         if t.dtype != torch.bfloat16:
-            raise TypeError(f"the grouped expert GEMMs run in bfloat16 (got {t.dtype}); cast the "
+            raise TypeError(f"the fused expert kernels run in bfloat16 (got {t.dtype}); cast the "
                             "module with .to(torch.bfloat16)")
+
+
+def _gemm_dtype(*tensors):
+    """bfloat16 (the tuned kernels) or float32 (the plain fp32 kernels) for all operands."""
+    dt = tensors[0].dtype
+    if dt not in (torch.bfloat16, torch.float32) or any(t.dtype != dt for t in tensors):
+        raise TypeError("the grouped expert GEMMs take operands that are all bfloat16 or all float32 "
+                        f"(got {[str(t.dtype) for t in tensors]})")
+    return dt
+
+
+def _grouped_gemm(kind, a, b, out, cum, rows, G, N, K, w_stride):
+    """om_grouped_gemm_{fwd,dgrad,wgrad}[_f32] by the operands' dtype."""
+    suffix = "_f32" if _gemm_dtype(a, b, out) == torch.float32 else ""
+    name = f"om_grouped_gemm_{kind}{suffix}"
+    _n.check(getattr(_n.lib(), name)(_n.ptr(a), _n.ptr(b), _n.ptr(out), _n.ptr(cum), rows, G, N, K,
+                                     w_stride, _n.stream()), name)
 
 
 # ----------------------------------------------------------------------------------------------
@@ -280,15 +297,14 @@ class GroupedGemmFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, merged_weight, cum_token_counts, max_tokens_per_expert=None,
                 use_triton_path=False):
-        _require_bf16(input, merged_weight)
+        _gemm_dtype(input, merged_weight)
         _n.require_cuda_contiguous(input)
         num_tokens = input.shape[0]
         num_experts, ofm, ifm = merged_weight.shape
         cum = _device_counts(cum_token_counts, input.device)
         output = torch.empty((num_tokens, ofm), dtype=input.dtype, device=input.device)
-        _n.check(_n.lib().om_grouped_gemm_fwd(
-            _n.ptr(input), _n.ptr(merged_weight), _n.ptr(output), _n.ptr(cum), num_tokens,
-            num_experts, ofm, ifm, _expert_stride(merged_weight), _n.stream()), "om_grouped_gemm_fwd")
+        _grouped_gemm("fwd", input, merged_weight, output, cum, num_tokens, num_experts, ofm, ifm,
+                      _expert_stride(merged_weight))
         ctx.save_for_backward(input, merged_weight, cum)
         return output
 
@@ -301,20 +317,17 @@ class GroupedGemmFunction(torch.autograd.Function):
         input_grad = torch.empty_like(input)
         merged_weight_grad = torch.empty((num_experts, ofm, ifm), dtype=merged_weight.dtype,
                                          device=merged_weight.device)
-        lib = _n.lib()
-        _n.check(lib.om_grouped_gemm_dgrad(
-            _n.ptr(output_grad), _n.ptr(merged_weight), _n.ptr(input_grad), _n.ptr(cum), rows,
-            num_experts, ofm, ifm, _expert_stride(merged_weight), _n.stream()), "om_grouped_gemm_dgrad")
-        _n.check(lib.om_grouped_gemm_wgrad(
-            _n.ptr(output_grad), _n.ptr(input), _n.ptr(merged_weight_grad), _n.ptr(cum), rows,
-            num_experts, ofm, ifm, 0, _n.stream()), "om_grouped_gemm_wgrad")
+        _grouped_gemm("dgrad", output_grad, merged_weight, input_grad, cum, rows, num_experts, ofm, ifm,
+                      _expert_stride(merged_weight))
+        _grouped_gemm("wgrad", output_grad, input, merged_weight_grad, cum, rows, num_experts, ofm, ifm, 0)
         return input_grad, merged_weight_grad, None, None, None
 
 
 def _merged_mlp_forward(x, w_gate, w_up, w_down, cum_token_counts, x_rows=None):
     """-> (y, cum, g, u, h).  Fused gate+up+SwiGLU launch, then the down projection.  With
     `x_rows` (int32 [rows]) the MLP input is x[x_rows] without that matrix being built."""
-    _require_bf16(x, w_gate, w_up, w_down)
+    if _gemm_dtype(x, w_gate, w_up, w_down) == torch.float32:
+        return _merged_mlp_forward_f32(x, w_gate, w_up, w_down, cum_token_counts, x_rows)
     _n.require_cuda_contiguous(x, x_rows)
     rows, H = x.shape
     if x_rows is not None:
@@ -345,9 +358,63 @@ def _merged_mlp_forward(x, w_gate, w_up, w_down, cum_token_counts, x_rows=None):
     return y, cum, g, u, h
 
 
+def _gathered_rows(x, x_rows):
+    if x_rows is None:
+        return x
+    out = torch.empty((x_rows.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    pcl_xpu_customops.index_gather(x, x_rows, out)
+    return out
+
+
+def _merged_mlp_forward_f32(x, w_gate, w_up, w_down, cum_token_counts, x_rows=None):
+    """float32 modules: the reference's own sequence (moe.py:396-405), three grouped GEMMs and the
+    SwiGLU glue kernel, on the plain fp32 kernels; nothing is fused."""
+    _n.require_cuda_contiguous(x, x_rows)
+    xs = _gathered_rows(x, x_rows)
+    rows, H = xs.shape
+    G, I, _ = w_gate.shape
+    cum = _device_counts(cum_token_counts, x.device)
+    g = torch.empty((rows, I), dtype=x.dtype, device=x.device)
+    u = torch.empty_like(g)
+    h = torch.empty_like(g)
+    y = torch.empty((rows, H), dtype=x.dtype, device=x.device)
+    with record_pcl_function("1moeblock--7gmlp_fwd"):
+        _grouped_gemm("fwd", xs, w_gate, g, cum, rows, G, I, H, _expert_stride(w_gate))
+        _grouped_gemm("fwd", xs, w_up, u, cum, rows, G, I, H, _expert_stride(w_up))
+        if rows:
+            _n.check(_n.lib().om_swiglu_fwd(_n.ptr(g), _n.ptr(u), _n.ptr(h), rows * I, _n.OM_F32, _n.stream()),
+                     "om_swiglu_fwd")
+        _grouped_gemm("fwd", h, w_down, y, cum, rows, G, H, I, _expert_stride(w_down))
+    return y, cum, g, u, h
+
+
+def _merged_mlp_backward_f32(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows=None):
+    dy = dy.contiguous()
+    xs = _gathered_rows(x, x_rows)
+    rows, H = dy.shape
+    G, I, _ = w_gate.shape
+    new = lambda *shape: torch.empty(shape, dtype=x.dtype, device=x.device)
+    dh, dg, du, dx, dx2 = new(rows, I), new(rows, I), new(rows, I), new(rows, H), new(rows, H)
+    dw_gate, dw_up, dw_down = new(G, I, H), new(G, I, H), new(G, H, I)
+    with record_pcl_function("1moeblock--7gmlp_bwd"):
+        _grouped_gemm("wgrad", dy, h, dw_down, cum, rows, G, H, I, 0)
+        _grouped_gemm("dgrad", dy, w_down, dh, cum, rows, G, H, I, _expert_stride(w_down))
+        if rows:
+            _n.check(_n.lib().om_swiglu_bwd(_n.ptr(dh), _n.ptr(g), _n.ptr(u), _n.ptr(dg), _n.ptr(du), rows * I,
+                                            _n.OM_F32, _n.stream()), "om_swiglu_bwd")
+        _grouped_gemm("wgrad", dg, xs, dw_gate, cum, rows, G, I, H, 0)
+        _grouped_gemm("wgrad", du, xs, dw_up, cum, rows, G, I, H, 0)
+        _grouped_gemm("dgrad", dg, w_gate, dx, cum, rows, G, I, H, _expert_stride(w_gate))
+        _grouped_gemm("dgrad", du, w_up, dx2, cum, rows, G, I, H, _expert_stride(w_up))
+        dx += dx2
+    return dx, dw_gate, dw_up, dw_down
+
+
 def _merged_mlp_backward(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows=None):
     """-> (dx, dw_gate [G,I,H], dw_up [G,I,H], dw_down [G,H,I]), all freshly allocated.  With
     `x_rows` the MLP input was x[x_rows]; dx is then the gradient of that gathered matrix."""
+    if x.dtype == torch.float32:
+        return _merged_mlp_backward_f32(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows)
     dy = dy.contiguous()
     rows, H = dy.shape
     G, I, _ = w_gate.shape

@@ -119,6 +119,14 @@ def test_grouped_gemms(lib):
     assert lib.om_merged_mlp_gate_up_fwd(P, P, None, P, P, P, P, 131072, 64, 1024, 2048, 0, None) == NULL
     assert lib.om_merged_mlp_down_dgrad(P, P, P, P, P, ODD, P, 131072, 64, 1024, 2048, 0, None) == ALIGN
     assert lib.om_merged_mlp_gate_up_dgrad(P, P, P, P, None, P, 131072, 64, 1024, 2048, 0, None) == NULL
+    # float32 forms: N, K multiples of 64
+    assert lib.om_grouped_gemm_fwd_f32(P, P, P, P, 4096, 8, 96, 256, 0, None) == SHAPE
+    assert lib.om_grouped_gemm_fwd_f32(P, P, P, P, 0, 8, 64, 256, 0, None) == OK
+    assert lib.om_grouped_gemm_fwd_f32(P, P, P, None, 4096, 8, 64, 256, 0, None) == NULL
+    assert lib.om_grouped_gemm_fwd_f32(P, P, P, P, 4096, 8, 64, 256, 64 * 256 + 2, None) == ALIGN   # pitch % 4
+    assert lib.om_grouped_gemm_dgrad_f32(P, ODD, P, P, 4096, 8, 64, 256, 0, None) == ALIGN
+    assert lib.om_grouped_gemm_wgrad_f32(P, P, None, P, 4096, 8, 64, 256, 0, None) == NULL
+    assert lib.om_grouped_gemm_wgrad_f32(P, P, P, P, 4096, 70000, 64, 256, 0, None) == SHAPE        # grid limit
     # the forms that read the tokens through an index
     g = (131072, 64, 1024, 2048, 0, None)
     assert lib.om_merged_mlp_gate_up_fwd_gathered(P, None, 16384, P, P, P, P, P, P, *g) == NULL      # no index

@@ -169,3 +169,40 @@ def test_gathered_merged_mlp_with_no_routed_rows(cuda):
     assert float(x.grad.abs().max()) == 0.0
     for w in ws:
         assert float(w.grad.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("kind,G,rows,N,K", [("uniform", 4, 512, 256, 128), ("ragged", 8, 1000, 192, 320),
+                                            ("empties", 16, 777, 64, 64), ("ragged", 3, 5, 128, 64),
+                                            ("uniform", 8, 4096, 512, 256)])
+def test_grouped_gemm_float32(cuda, kind, G, rows, N, K):
+    """float32 modules (the reference's GroupedGemmFunction runs in the module's dtype): the fp32
+    kernels against per-expert matmul in float64.  fp32 products and sums, so only the order of
+    summation differs from torch's fp32 matmul: errors of a few fp32 roundings of the absolute sum."""
+    from optimus.models.common.moe import GroupedGemmFunction
+    g = torch.Generator().manual_seed(rows + 7)
+    x = torch.randn(rows, K, generator=g)
+    w = torch.randn(G, N, K, generator=g) * 0.05
+    dout = torch.randn(rows, N, generator=g)
+    cum = _counts(kind, G, rows)
+    xd = x.to(cuda).requires_grad_(True)
+    wd = w.to(cuda).requires_grad_(True)
+    out = GroupedGemmFunction.apply(xd, wd, cum, int((cum[1:] - cum[:-1]).max()), False)
+    assert out.dtype == torch.float32
+    out.backward(dout.to(cuda))
+    X, W, D = x.double(), w.double(), dout.double()
+    ref = torch.zeros(rows, N, dtype=torch.float64)
+    dx_ref = torch.zeros(rows, K, dtype=torch.float64)
+    dw_ref = torch.zeros(G, N, K, dtype=torch.float64)
+    ref_abs, dx_abs, dw_abs = torch.zeros_like(ref), torch.zeros_like(dx_ref), torch.zeros_like(dw_ref)
+    for e in range(G):
+        s, t = int(cum[e]), int(cum[e + 1])
+        ref[s:t] = X[s:t] @ W[e].t(); ref_abs[s:t] = X[s:t].abs() @ W[e].abs().t()
+        dx_ref[s:t] = D[s:t] @ W[e]; dx_abs[s:t] = D[s:t].abs() @ W[e].abs()
+        dw_ref[e] = D[s:t].t() @ X[s:t]; dw_abs[e] = D[s:t].abs().t() @ X[s:t].abs()
+    for name, got, want, scale in (("out", out, ref, ref_abs), ("dx", xd.grad, dx_ref, dx_abs),
+                                   ("dw", wd.grad, dw_ref, dw_abs)):
+        err = (got.detach().double().cpu() - want).abs()
+        assert bool((err <= 2e-6 * scale + 1e-30).all()), (name, float((err / (scale + 1e-30)).max()))
+    empty = (cum[1:] == cum[:-1])
+    if empty.any():
+        assert float(wd.grad[empty.to(cuda)].abs().max()) == 0.0

@@ -121,6 +121,56 @@ def test_fast_block_odd_small_shapes(cuda, T, H, I, N, K, renorm):
         assert max_abs(a, gref) <= MAX_ABS * max(1.0, float(gref.abs().max())), (k, max_abs(a, gref))
 
 
+@pytest.mark.parametrize("merged", [True, False])
+def test_fast_block_float32_c1(cuda, merged):
+    """BASELINE's first configuration as the reference states it: a float32 module.  The router, the
+    index construction, the row kernels and the fp32 grouped GEMMs all run in float32, so the bar is
+    fp32 accuracy (summation order only), not the bf16 one."""
+    inp = sc.moe_inputs("C1")
+    c = inp["cfg"]
+    f32 = {k: (v.float() if torch.is_tensor(v) else v) for k, v in inp.items()}
+    ref_out, ref_logits, ref_grads = _reference({k: (v.clone() if torch.is_tensor(v) else v) for k, v in f32.items()})
+    from optimus.mapper import ParallelDpPpEpTpMapper
+    from optimus.models.common.moe import FastOlmoeParallelSparseMoeBlock
+    from optimus.models.olmoe.configuration_olmoe import OlmoeParallelConfig
+    cfg = OlmoeParallelConfig(hidden_size=c["H"], intermediate_size=c["I"], num_experts=c["N"],
+                              num_experts_per_tok=c["K"], norm_topk_prob=c["norm_topk_prob"],
+                              output_router_logits=True, use_fast_moe=True, use_merged_mlp_in_fast_moe=merged)
+    blk = FastOlmoeParallelSparseMoeBlock(cfg, ParallelDpPpEpTpMapper()).to(cuda)      # stays float32
+    with torch.no_grad():
+        blk.gate.weight.copy_(f32["gate_w"])
+        if merged:
+            blk.experts.gate_proj_merged_weight.copy_(f32["w_gate"])
+            blk.experts.up_proj_merged_weight.copy_(f32["w_up"])
+            blk.experts.down_proj_merged_weight.copy_(f32["w_down"])
+        else:
+            for e, m in enumerate(blk.experts):
+                m.gate_proj.weight.copy_(f32["w_gate"][e]); m.up_proj.weight.copy_(f32["w_up"][e])
+                m.down_proj.weight.copy_(f32["w_down"][e])
+    x = f32["x"].to(cuda).view(1, c["T"], c["H"]).requires_grad_(True)
+    out, logits = blk(x)
+    assert out.dtype == torch.float32
+    out.backward(f32["dout"].to(cuda).view_as(out))
+    _, e_ref, _ = R.olmoe_router(ref_logits, c["K"], c["norm_topk_prob"], torch.float32)
+    _, e_gpu, _ = R.olmoe_router(logits.float().cpu(), c["K"], c["norm_topk_prob"], torch.float32)
+    assert torch.equal(e_ref, e_gpu)
+    o = out.detach().cpu().view(c["T"], c["H"])
+    assert max_abs(o, ref_out) <= 1e-5 * max(1.0, float(ref_out.abs().max())) and mean_rel(o, ref_out) <= 1e-5
+    if merged:
+        got = {"x": x.grad.view(c["T"], c["H"]), "gate_w": blk.gate.weight.grad,
+               "w_gate": blk.experts.gate_proj_merged_weight.grad, "w_up": blk.experts.up_proj_merged_weight.grad,
+               "w_down": blk.experts.down_proj_merged_weight.grad}
+    else:
+        got = {"x": x.grad.view(c["T"], c["H"]), "gate_w": blk.gate.weight.grad,
+               "w_gate": torch.stack([m.gate_proj.weight.grad for m in blk.experts]),
+               "w_up": torch.stack([m.up_proj.weight.grad for m in blk.experts]),
+               "w_down": torch.stack([m.down_proj.weight.grad for m in blk.experts])}
+    for k, gref in ref_grads.items():
+        a = got[k].float().cpu()
+        assert mean_rel(a, gref) <= 2e-5, (k, mean_rel(a, gref))
+        assert max_abs(a, gref) <= 1e-4 * max(1.0, float(gref.abs().max())), (k, max_abs(a, gref))
+
+
 def test_fast_block_injected_logits_skewed(cuda):
     """C4: Zipf-skewed routing injected at the functional level (router logits given): many experts
     get 0-8 rows, a few get hundreds.  Expert computation only (router excluded), fwd+bwd."""
