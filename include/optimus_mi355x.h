@@ -247,6 +247,19 @@ int om_reduce_ggemm_output(const void *ggemm_output, const void *routing_weights
                            const int32_t *selected_experts_indices, const int32_t *output_indices,
                            void *final_hidden_states, int64_t T, int K, int64_t E, int dtype,
                            int weights_dtype, int skip_weights_scaling, void *stream);
+/* om_reduce_ggemm_output_residual: the combine with the addition that follows it in the callers
+ * folded in,
+ *   final[t,:] = residual[t,:] + round(sum_i w * ggemm_output[...])     (sum rounded to `dtype` first,
+ * so the two roundings of the reference's two steps are both there): the decoder layer's
+ *   hidden_states = residual + hidden_states     (optimus/models/olmoe/modeling_olmoe.py:415)
+ * and the DeepSeek-V3 block's routed + shared-expert sum (modeling_deepseek_v3.py:265).
+ * residual [T,E] of `dtype`; may alias nothing else.                                          */
+int om_reduce_ggemm_output_residual(const void *ggemm_output, const void *routing_weights,
+                                    const int32_t *cum_expert_counts_ep,
+                                    const int32_t *selected_experts_indices,
+                                    const int32_t *output_indices, const void *residual,
+                                    void *final_hidden_states, int64_t T, int K, int64_t E,
+                                    int dtype, int weights_dtype, void *stream);
 int om_reduce_ggemm_output_backward(const void *final_hidden_states_grad, const void *ggemm_output,
                                     const void *routing_weights,
                                     const int32_t *selected_experts_indices,

@@ -30,20 +30,29 @@ __global__ __launch_bounds__(256) void index_gather_kernel(const T *__restrict__
     }
 }
 
+// out = residual + round_to_T(sum): the two roundings of `residual + moe_output` on tensors of type T
+template <typename T> __device__ __forceinline__ float round_as(float x);
+template <> __device__ __forceinline__ float round_as<float>(float x) { return x; }
+template <> __device__ __forceinline__ float round_as<uint16_t>(float x) {
+    return bf16_bits_to_f32(f32_to_bf16_bits(x));
+}
+
 // hidden_grad[t,:] = sum_i ggemm_input_grad[output_indices[i],:],  i in [cum_ep[t], cum_ep[t+1])
 // SCALE: final[t,:] = sum_i w[t, sel_idx[i]] * y[output_indices[i],:]
+// residual != null: final[t,:] = residual[t,:] + T(that sum), the sum rounded to T first
 template <typename T, typename TW, bool SCALE>
 __global__ __launch_bounds__(256) void token_reduce_kernel(
     const T *__restrict__ rows, const TW *__restrict__ routing_weights,
     const int32_t *__restrict__ cum_expert_counts_ep,
     const int32_t *__restrict__ selected_experts_indices,
     const int32_t *__restrict__ output_indices, T *__restrict__ out, int64_t T_tokens, int K,
-    int64_t E, bool vec_ok) {
+    int64_t E, bool vec_ok, const T *__restrict__ residual = nullptr) {
     const int lane = threadIdx.x & 63;
     const int64_t t = static_cast<int64_t>(blockIdx.x) * ROWS_PER_BLOCK + (threadIdx.x >> 6);
     if (t >= T_tokens) return;
     const int32_t i0 = cum_expert_counts_ep[t], i1 = cum_expert_counts_ep[t + 1];
     T *dst = out + t * E;
+    const T *res = residual ? residual + t * E : nullptr;
     constexpr int V = Elem<T>::VEC;
     if (vec_ok) {
         // The token's row numbers and weights are fetched once, 64 at a time, one per lane, and
@@ -89,7 +98,14 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
 #pragma unroll
             for (int u = 0; u < CH; u++) {
                 const int64_t c = c0 + u * 64 + lane;
-                if (c < nv) reinterpret_cast<u32x4 *>(dst)[c] = Elem<T>::pack(acc[u]);
+                if (c >= nv) continue;
+                if (res) {
+                    float r[V];
+                    Elem<T>::unpack(reinterpret_cast<const u32x4 *>(res)[c], r);
+#pragma unroll
+                    for (int j = 0; j < V; j++) acc[u][j] = r[j] + round_as<T>(acc[u][j]);
+                }
+                reinterpret_cast<u32x4 *>(dst)[c] = Elem<T>::pack(acc[u]);
             }
         }
     } else {
@@ -102,6 +118,7 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
                 const float f = Elem<T>::load(rows + static_cast<int64_t>(index) * E + e);
                 acc += SCALE ? (f * scaling) : f;
             }
+            if (res) acc = Elem<T>::load(res + e) + round_as<T>(acc);
             Elem<T>::store(dst + e, acc);
         }
     }
@@ -247,12 +264,13 @@ extern "C" int om_shuffle_sub_matrix_reduce(const void *ggemm_input_grad,
     return om_launch_status();
 }
 
-extern "C" int om_reduce_ggemm_output(const void *ggemm_output, const void *routing_weights,
+namespace {
+int reduce_ggemm_output_launch(const void *ggemm_output, const void *routing_weights,
                                       const int32_t *cum_expert_counts_ep,
                                       const int32_t *selected_experts_indices,
                                       const int32_t *output_indices, void *final_hidden_states,
                                       int64_t T, int K, int64_t E, int dtype, int weights_dtype,
-                                      int skip_weights_scaling, void *stream) {
+                                      int skip_weights_scaling, const void *residual, void *stream) {
     if (dtype != OM_F32 && dtype != OM_BF16) return OM_ERR_DTYPE;
     if (weights_dtype != OM_F32 && weights_dtype != OM_BF16) return OM_ERR_DTYPE;
     if (dtype == OM_F32 && weights_dtype != OM_F32) return OM_ERR_DTYPE;
@@ -267,7 +285,8 @@ extern "C" int om_reduce_ggemm_output(const void *ggemm_output, const void *rout
         static_cast<const TT *>(ggemm_output), static_cast<const TW *>(routing_weights),           \
         cum_expert_counts_ep, selected_experts_indices, output_indices,                            \
         static_cast<TT *>(final_hidden_states), T, K, E,                                           \
-        row_vec_ok<TT>(ggemm_output, final_hidden_states, nullptr, E))
+        row_vec_ok<TT>(ggemm_output, final_hidden_states, residual, E),                           \
+        static_cast<const TT *>(residual))
     if (skip_weights_scaling) {
         if (dtype == OM_F32) OM_REDUCE(float, float, false);
         else OM_REDUCE(uint16_t, float, false);
@@ -280,6 +299,30 @@ extern "C" int om_reduce_ggemm_output(const void *ggemm_output, const void *rout
     }
 #undef OM_REDUCE
     return om_launch_status();
+}
+}  // namespace
+
+extern "C" int om_reduce_ggemm_output(const void *ggemm_output, const void *routing_weights,
+                                      const int32_t *cum_expert_counts_ep,
+                                      const int32_t *selected_experts_indices,
+                                      const int32_t *output_indices, void *final_hidden_states,
+                                      int64_t T, int K, int64_t E, int dtype, int weights_dtype,
+                                      int skip_weights_scaling, void *stream) {
+    return reduce_ggemm_output_launch(ggemm_output, routing_weights, cum_expert_counts_ep,
+                                      selected_experts_indices, output_indices, final_hidden_states, T, K,
+                                      E, dtype, weights_dtype, skip_weights_scaling, nullptr, stream);
+}
+
+extern "C" int om_reduce_ggemm_output_residual(const void *ggemm_output, const void *routing_weights,
+                                               const int32_t *cum_expert_counts_ep,
+                                               const int32_t *selected_experts_indices,
+                                               const int32_t *output_indices, const void *residual,
+                                               void *final_hidden_states, int64_t T, int K, int64_t E,
+                                               int dtype, int weights_dtype, void *stream) {
+    if (T > 0 && E > 0 && !residual) return OM_ERR_NULL;
+    return reduce_ggemm_output_launch(ggemm_output, routing_weights, cum_expert_counts_ep,
+                                      selected_experts_indices, output_indices, final_hidden_states, T, K,
+                                      E, dtype, weights_dtype, 0, residual, stream);
 }
 
 extern "C" int om_reduce_ggemm_output_backward(

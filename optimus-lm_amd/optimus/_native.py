@@ -70,6 +70,8 @@ SIGNATURES = {
                                              c_int, c_void_p]),
     "om_reduce_ggemm_output": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                        c_i64, c_int, c_i64, c_int, c_int, c_int, c_void_p]),
+    "om_reduce_ggemm_output_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                c_void_p, c_i64, c_int, c_i64, c_int, c_int, c_void_p]),
     "om_reduce_ggemm_output_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                 c_void_p, c_void_p, c_void_p, c_i64, c_int, c_i64,
                                                 c_int, c_int, c_void_p]),

@@ -676,6 +676,33 @@ class GroupGemmOutputReductionFunction(torch.autograd.Function):
         return ggemm_output_grad, routing_weights_grad, None, None, None, None, None, None, None, None
 
 
+class GroupGemmOutputReductionResidualFunction(torch.autograd.Function):
+    """residual + GroupGemmOutputReductionFunction(...) in one pass: the combined sum is rounded to
+    the activation dtype and then added to `residual` (both roundings of the two-step form).  Used
+    for the decoder layer's residual connection (modeling_olmoe.py:415) and for the DeepSeek-V3
+    block's routed + shared sum (modeling_deepseek_v3.py:265).  The gradient of the output goes to
+    `residual` unchanged and into the combine's backward."""
+
+    @staticmethod
+    def forward(ctx, ggemm_output, routing_weights, cum_expert_counts_ep, selected_experts_indices,
+                input_indices, output_indices, residual):
+        routing_weights = routing_weights.contiguous()
+        residual = residual.contiguous()
+        ctx.save_for_backward(ggemm_output, routing_weights, cum_expert_counts_ep,
+                              selected_experts_indices, input_indices, output_indices)
+        with record_pcl_function("1moeblock--8gmlp_output_reduction_fwd"):
+            final_hidden_states = torch.empty_like(residual)
+            pcl_xpu_customops.reduce_ggemm_output_residual(
+                ggemm_output, routing_weights, cum_expert_counts_ep, selected_experts_indices,
+                output_indices, residual, final_hidden_states)
+        return final_hidden_states
+
+    @staticmethod
+    def backward(ctx, final_hidden_states_grad):
+        grads = GroupGemmOutputReductionFunction.backward(ctx, final_hidden_states_grad)
+        return grads[0], grads[1], None, None, None, None, final_hidden_states_grad
+
+
 # ----------------------------------------------------------------------------------------------
 # Modules
 # ----------------------------------------------------------------------------------------------
@@ -708,11 +735,13 @@ class MergedMLP(nn.Module):
 
 
 def expert_computation(hidden_states, routing_weights, selected_experts, expert_start_idx,
-                       expert_end_idx, experts_fn, num_total_experts, gathered_experts_fn=None):
+                       expert_end_idx, experts_fn, num_total_experts, gathered_experts_fn=None,
+                       residual=None):
     """K1..K6 for 2-D hidden_states [T,H]: permute, run `experts_fn(ggemm_input, cum_token_counts)`,
     combine.  Shared by the OLMoE and DeepSeek-V3 blocks.  With `gathered_experts_fn(hidden_states,
     input_indices, cum_expert_counts_ep, output_indices, cum_token_counts)` the experts read the
-    tokens through the index and K4's gathered copy is not built."""
+    tokens through the index and K4's gathered copy is not built.  With `residual` [T,H] the result
+    is residual + combine(...), added inside the combine kernel."""
     T, K = selected_experts.shape
     with record_pcl_function("1moeblock--3index_calculation"):
         (cum_token_counts, cum_expert_counts_ep, input_indices, output_indices,
@@ -732,6 +761,10 @@ def expert_computation(hidden_states, routing_weights, selected_experts, expert_
         ggemm_input = PrepareInputForGroupGemmFunction.apply(hidden_states, input_indices,
                                                              cum_expert_counts_ep, output_indices)
         ggemm_output = experts_fn(ggemm_input, cum_token_counts)
+    if residual is not None:
+        return GroupGemmOutputReductionResidualFunction.apply(
+            ggemm_output, routing_weights, cum_expert_counts_ep, selected_experts_indices, input_indices,
+            output_indices, residual)
     return GroupGemmOutputReductionFunction.apply(ggemm_output, routing_weights, cum_expert_counts_ep,
                                                   selected_experts_indices, input_indices,
                                                   output_indices)
@@ -796,7 +829,13 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
         return GatheredGroupMLPFunction.apply(hidden_states, input_indices, cum_expert_counts_ep,
                                               output_indices, cum_token_counts, *mlp_params)
 
-    def forward(self, hidden_states):
+    def forward_with_residual(self, hidden_states, residual):
+        """(residual + forward(hidden_states)[0], router_logits): the decoder layer's
+        `hidden_states = residual + hidden_states` after the block (modeling_olmoe.py:415) folded into
+        the combine kernel; same bits as the two steps."""
+        return self.forward(hidden_states, residual=residual)
+
+    def forward(self, hidden_states, residual=None):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
         flat = hidden_states.reshape(-1, hidden_dim)
         if self.router_logits_fp32 and gate_kernel_fits(flat, self.gate.weight):
@@ -812,15 +851,18 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
                 router_logits.contiguous(), self.num_experts_per_tok, self.norm_topk_prob,
                 hidden_states.dtype)
 
-        def expert_computation_block(hidden_states, selected_experts, routing_weights):
+        def expert_computation_block(hidden_states, selected_experts, routing_weights, residual=None):
             b, s, h = hidden_states.shape
             gathered = self._gathered_experts_fn if self.fuse_input_gather else None
             out = expert_computation(hidden_states.reshape(-1, h), routing_weights, selected_experts,
                                      self.expert_start_idx, self.expert_end_idx, self._experts_fn,
-                                     self.num_experts, gathered_experts_fn=gathered)
+                                     self.num_experts, gathered_experts_fn=gathered,
+                                     residual=None if residual is None else residual.reshape(-1, h))
             return out.reshape(b, s, h)
 
         args = [hidden_states, selected_experts, routing_weights]
+        if residual is not None:
+            args.append(residual)
         if self.use_activation_checkpointing_for_moe:
             final_hidden_states = torch_activation_checkpoint(expert_computation_block, *args,
                                                               use_reentrant=False)

@@ -149,14 +149,16 @@ class DeepseekV3ParallelMoE(nn.Module):
         return _moe.GatheredGroupMLPFunction.apply(hidden_states, input_indices, cum_expert_counts_ep,
                                                    output_indices, cum_token_counts, *params)
 
-    def moe(self, hidden_states, topk_indices, topk_weights):
+    def moe(self, hidden_states, topk_indices, topk_weights, residual=None):
         """Routed part for [T,H] hidden_states (reference :221-244): fp32 weights, fp32 sum over a
         token's local experts, one rounding to the activation dtype.  The local experts read their
-        tokens through the permutation index (no gathered copy of the activations)."""
+        tokens through the permutation index (no gathered copy of the activations).  `residual`
+        [T,H] is added to the rounded result inside the combine kernel."""
         gathered = self._gathered_experts_fn if getattr(self.config, "fuse_input_gather", True) else None
         return _moe.expert_computation(hidden_states, topk_weights, topk_indices,
                                        self.expert_start_idx, self.expert_end_idx, self._experts_fn,
-                                       self.config.n_routed_experts, gathered_experts_fn=gathered)
+                                       self.config.n_routed_experts, gathered_experts_fn=gathered,
+                                       residual=residual)
 
     def forward(self, hidden_states):
         topk_indices, topk_weights = self.gate(hidden_states)
@@ -165,8 +167,11 @@ class DeepseekV3ParallelMoE(nn.Module):
             residuals = hidden_states
             orig_shape = hidden_states.shape
             flat = hidden_states.reshape(-1, hidden_states.shape[-1])
-            final_hidden_states = self.moe(flat, topk_indices, topk_weights).view(*orig_shape)
-            return final_hidden_states + self.shared_experts(residuals)
+            # routed + shared (reference :265): the shared experts' output goes into the combine
+            # kernel as its residual, which rounds the routed sum first and then adds: the same two
+            # roundings as `moe(...) + shared_experts(...)`
+            shared = self.shared_experts(residuals).reshape(flat.shape)
+            return self.moe(flat, topk_indices, topk_weights, residual=shared).view(*orig_shape)
 
         args = [hidden_states, topk_indices, topk_weights]
         if self.use_activation_checkpointing_for_moe:

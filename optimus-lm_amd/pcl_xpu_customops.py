@@ -98,6 +98,22 @@ def reduce_ggemm_output(ggemm_output, routing_weights, cum_expert_counts_ep,
         int(bool(skip_weights_scaling)), _n.stream()), "reduce_ggemm_output")
 
 
+def reduce_ggemm_output_residual(ggemm_output, routing_weights, cum_expert_counts_ep,
+                                 selected_experts_indices, output_indices, residual, final_hidden_states):
+    """K6 forward with the addition that follows it folded in: final = residual + combine(...),
+    the combined sum rounded to the activation dtype before the addition (not in the reference's
+    module; see om_reduce_ggemm_output_residual)."""
+    _n.require_cuda_contiguous(ggemm_output, routing_weights, cum_expert_counts_ep,
+                               selected_experts_indices, output_indices, residual, final_hidden_states)
+    T, K = routing_weights.shape
+    E = ggemm_output.shape[1]
+    _n.check(_n.lib().om_reduce_ggemm_output_residual(
+        _n.ptr(ggemm_output), _n.ptr(routing_weights), _n.ptr(cum_expert_counts_ep),
+        _n.ptr(selected_experts_indices), _n.ptr(output_indices), _n.ptr(residual),
+        _n.ptr(final_hidden_states), T, K, E, _n.dtype_code(ggemm_output),
+        _n.dtype_code(routing_weights), _n.stream()), "reduce_ggemm_output_residual")
+
+
 def reduce_ggemm_output_backward(final_hidden_states_grad, ggemm_output, routing_weights,
                                  cum_expert_counts_ep, selected_experts_indices, input_indices,
                                  output_indices, ggemm_output_grad, routing_weights_grad):

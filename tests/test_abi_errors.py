@@ -105,6 +105,14 @@ def test_rmsnorm_and_balance(lib):
     assert lib.om_router_balance_bwd(P, F32, None, 1000, 64, P, None) == NULL
 
 
+def test_combine_with_residual(lib):
+    args = (16384, 8, 2048, BF16, BF16, None)
+    assert lib.om_reduce_ggemm_output_residual(P, P, P, P, P, None, P, *args) == NULL        # no residual
+    assert lib.om_reduce_ggemm_output_residual(P, P, P, P, P, P, None, *args) == NULL
+    assert lib.om_reduce_ggemm_output_residual(P, P, P, P, P, P, P, 16384, 8, 2048, 7, BF16, None) == DTYPE
+    assert lib.om_reduce_ggemm_output_residual(P, P, P, P, P, None, P, 0, 8, 2048, BF16, BF16, None) == OK
+
+
 def test_grouped_gemms(lib):
     args = (131072, 64, 2048, 1024, 0, None)
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 131072, 64, 2000, 1024, 0, None) == SHAPE    # N % 128

@@ -308,6 +308,29 @@ def test_block_whose_expert_window_gets_no_token(cuda, merged):
         assert p.grad is not None and float(p.grad.abs().max()) == 0.0
 
 
+def test_block_with_residual_equals_block_plus_add(cuda):
+    """forward_with_residual folds the decoder layer's `residual + moe_output` into the combine
+    kernel: output and all gradients equal the two-step form bit for bit."""
+    inp = sc.moe_inputs("C1", scale_tokens=0.5)
+    c = inp["cfg"]
+    g = torch.Generator().manual_seed(9)
+    res0 = torch.randn(1, c["T"], c["H"], generator=g).to(torch.bfloat16)
+    results = []
+    for fused in (True, False):
+        blk = _olmoe_block(inp, cuda)
+        x = inp["x"].to(cuda).view(1, c["T"], c["H"]).requires_grad_(True)
+        r = res0.to(cuda).requires_grad_(True)
+        if fused:
+            out, _ = blk.forward_with_residual(x, r)
+        else:
+            out = r + blk(x)[0]
+        out.backward(inp["dout"].to(cuda).view_as(out))
+        results.append([out.detach(), x.grad, r.grad] + [p.grad for p in blk.parameters()])
+    for a0, a1 in zip(*results):
+        assert torch.equal(a0, a1)
+    assert torch.equal(results[0][2], inp["dout"].to(cuda).view_as(results[0][2]))
+
+
 @pytest.mark.parametrize("ep_ind", [0, 3])
 def test_dsv3_block_one_rank_share(cuda, ep_ind):
     """C5 at reduced size: DeepseekV3ParallelMoE with expert_parallelism=8 (32 of 256 routed experts

@@ -93,3 +93,25 @@ def test_index_add_and_autograd_function(cuda, oracle_lib, dtype):
     gout = torch.randn(S, E, generator=g).to(dtype).to(cuda)
     res.backward(gout)
     assert torch.equal(eo.grad, gout[uniq.long().to(cuda)])
+
+
+@pytest.mark.parametrize("dtype,wdtype", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                          (torch.float32, torch.float32)])
+@pytest.mark.parametrize("T,N,K,E,start,end", [(64, 8, 2, 256, 0, 8), (512, 64, 8, 2048, 0, 64),
+                                              (256, 32, 4, 136, 8, 24), (128, 8, 2, 100, 0, 8)])
+def test_combine_with_residual_equals_two_steps(cuda, oracle_lib, dtype, wdtype, T, N, K, E, start, end):
+    """reduce_ggemm_output_residual = reduce_ggemm_output (already bit-exact against the restatement
+    of the SYCL kernel) followed by the tensor addition the callers perform: the same bits, for an
+    expert window (tokens without a local expert get residual + 0) and row lengths that are not a
+    multiple of the vector width."""
+    import pcl_xpu_customops as ops
+    se, idx, x, y, w = _setup(T, N, K, E, start, end, dtype, oracle_lib, seed=5)
+    d = lambda a: torch.from_numpy(a).to(cuda)
+    oi, si, ce = d(idx["output_indices"]), d(idx["selected_experts_indices"]), d(idx["cum_expert_counts_ep"])
+    yd, wd, res = y.to(cuda), w.to(wdtype).to(cuda), x.to(cuda)
+    two = torch.empty(T, E, dtype=dtype, device=cuda)
+    ops.reduce_ggemm_output(yd, wd, ce, si, oi, two, False)
+    two = res + two
+    one = torch.empty(T, E, dtype=dtype, device=cuda)
+    ops.reduce_ggemm_output_residual(yd, wd, ce, si, oi, res, one)
+    assert np.array_equal(bits(one), bits(two))
