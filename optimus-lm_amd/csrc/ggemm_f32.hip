@@ -26,7 +26,7 @@ struct F32Params {
     float *C;
     const int32_t *cum;
     int64_t lda, ldb, ldc, strideB, strideC;
-    int n_experts, n_cols, kc, m_tiles_max;
+    int n_experts, n_cols, kc;
 };
 
 // Fill tile[row][c] (64 x 16) from an operand.  CONTIG: element (row, c) at base[(r0+row)*ld + c0+c],
