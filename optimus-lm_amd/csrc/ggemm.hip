@@ -735,8 +735,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 
 // ---- host side ---------------------------------------------------------------------------------
 
-// Two tile shapes: 256x256 (wavefront tile 128x128) for the training shapes, 128x128 (wavefront
-// tile 64x64) when an extent is not a multiple of 256 or experts hold few rows each.
+// Two tile shapes: 256x256 (8 wavefronts of 128x64) for the training shapes, 128x128 (4 wavefronts
+// of 64x64) when an extent is not a multiple of 256 or experts hold few rows each.
 
 inline bool mult(int64_t v, int m) { return v > 0 && v % m == 0; }
 inline bool fits31(int64_t elems) { return elems >= 0 && elems < (1LL << 31); }
