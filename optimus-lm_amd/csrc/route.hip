@@ -15,13 +15,61 @@ template <typename T> __device__ __forceinline__ float load_logit(const T *p);
 template <> __device__ __forceinline__ float load_logit<float>(const float *p) { return *p; }
 template <> __device__ __forceinline__ float load_logit<uint16_t>(const uint16_t *p) { return bf16_bits_to_f32(*p); }
 
-// (value, index) arg-max across the wavefront; ties go to the lower index.
-__device__ __forceinline__ void wave_argmax(float &v, int &i) {
+// (value, index) arg-max across the wavefront by an xor butterfly of lane permutes; ties go to
+// the lower index.  Twelve dependent permutes: the slow path of wave_argmax below.
+__device__ __forceinline__ void wave_argmax_butterfly(float &v, int &i) {
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(v, o, 64);
         const int oi = __shfl_xor(i, o, 64);
         if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
     }
+}
+
+// Maximum over the wavefront with data-parallel-primitive moves (no LDS traffic): within each row
+// of 16 lanes by quad permutes and mirrors, then row 0 -> 1 and 2 -> 3, then rows 0-1 -> 2-3; lane
+// 63 ends with the maximum and hands it to everyone through a scalar register.  A maximum does not
+// depend on the order of the comparisons, so this is exact.
+__device__ __forceinline__ float wave_max_dpp(float v) {
+    int x = __float_as_int(v);
+#define OM_DPP_MAX(ctrl, row_mask)                                                                   \
+    x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(         \
+            x, x, ctrl, row_mask, 0xf, false))))
+    OM_DPP_MAX(0xB1, 0xf);    // quad_perm [1,0,3,2]
+    OM_DPP_MAX(0x4E, 0xf);    // quad_perm [2,3,0,1]
+    OM_DPP_MAX(0x141, 0xf);   // row_half_mirror
+    OM_DPP_MAX(0x140, 0xf);   // row_mirror: every lane of a row holds the row's maximum
+    OM_DPP_MAX(0x142, 0xa);   // row_bcast15 into rows 1 and 3
+    OM_DPP_MAX(0x143, 0xc);   // row_bcast31 into rows 2 and 3
+#undef OM_DPP_MAX
+    return __int_as_float(__builtin_amdgcn_readlane(x, 63));
+}
+
+// (value, index) arg-max across the wavefront; ties go to the lower index.  Fast path: the maximum
+// by wave_max_dpp, a ballot of the lanes that hold it, and when exactly one lane does (no tie, no
+// NaN) its index through a scalar lane read.  Everything else takes the butterfly, so the result
+// is the butterfly's in every case.
+__device__ __forceinline__ void wave_argmax(float &v, int &i) {
+    const float m = wave_max_dpp(v);
+    const unsigned long long vote = __ballot(v == m);
+    if (__popcll(vote) == 1) {
+        const int src = __ffsll(static_cast<long long>(vote)) - 1;
+        i = __builtin_amdgcn_readlane(i, src);
+        v = m;
+    } else {
+        wave_argmax_butterfly(v, i);
+    }
+}
+
+// value of `x[e / 64]` held by lane e % 64, for a per-lane e (e < 0: undefined, caller masks)
+template <int PER>
+__device__ __forceinline__ float fetch_expert_value(const float (&x)[PER], int e) {
+    float out = 0.0f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const float v = __shfl(x[j], e & 63, 64);
+        if ((e >> 6) == j) out = v;
+    }
+    return out;
 }
 
 // softmax probabilities of this token's row into p[PER]; returns nothing else.
@@ -34,7 +82,7 @@ __device__ __forceinline__ void row_softmax(const T *row, int N, int lane, float
         p[j] = (i < N) ? load_logit<T>(row + i) : -INFINITY;
         mx = fmaxf(mx, p[j]);
     }
-    mx = wave_max(mx);
+    mx = wave_max_dpp(mx);
     float sum = 0.0f;
 #pragma unroll
     for (int j = 0; j < PER; j++) {
@@ -108,16 +156,8 @@ __global__ __launch_bounds__(256) void softmax_topk_bwd_kernel(const T *__restri
     // lane k < K: its expert, the probability there and the incoming gradient
     const int e = (lane < K) ? static_cast<int>(experts[t * K + lane]) : -1;
     float dwk = (lane < K) ? Elem<TW>::load(dweights + t * K + lane) : 0.0f;
-    float wk = 0.0f;
-    for (int k = 0; k < K; k++) {
-        const int ek = __shfl(e, k, 64);
-        float pv = 0.0f;
-#pragma unroll
-        for (int j = 0; j < PER; j++)
-            if (lane + 64 * j == ek) pv = p[j];
-        pv = wave_sum(pv);  // exactly one lane holds it
-        if (lane == k) wk = pv;
-    }
+    float wk = fetch_expert_value<PER>(p, e);   // lane k < K: the probability of its expert
+    if (lane >= K) wk = 0.0f;
     if (renorm) {
         const float S = wave_sum(wk);
         const float dot = wave_sum(dwk * wk);
@@ -198,16 +238,8 @@ __global__ __launch_bounds__(256) void sigmoid_group_topk_kernel(
     float cv; int e;
     select_topk<PER>(choice, N, K, lane, cv, e);
     // weight = sigmoid score (no bias) at the selected expert
-    float w = 0.0f;
-    for (int k = 0; k < K; k++) {
-        const int ek = __shfl(e, k, 64);
-        float sv = 0.0f;
-#pragma unroll
-        for (int j = 0; j < PER; j++)
-            if (lane + 64 * j == ek) sv = score[j];
-        sv = wave_sum(sv);
-        if (lane == k) w = sv;
-    }
+    float w = fetch_expert_value<PER>(score, e);
+    if (lane >= K) w = 0.0f;
     if (renorm) {
         const float S = wave_sum(lane < K ? w : 0.0f) + 1e-20f;
         w = w / S;
