@@ -206,3 +206,40 @@ def test_grouped_gemm_float32(cuda, kind, G, rows, N, K):
     empty = (cum[1:] == cum[:-1])
     if empty.any():
         assert float(wd.grad[empty.to(cuda)].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("seed", list(range(24)))
+def test_grouped_gemm_random_shapes(cuda, seed):
+    """Seeded sweep over expert counts, row counts and sizes: exercises the persistent-block
+    partition (fewer tiles than blocks, remainders over the 8 XCDs, experts without rows, one or many
+    tiles per expert) on both tile shapes, against per-expert fp32 matmul."""
+    from optimus.models.common.moe import GroupedGemmFunction
+    rng = np.random.RandomState(1234 + seed)
+    G = int(rng.choice([1, 2, 3, 7, 16, 33, 64, 70]))
+    rows = int(rng.choice([1, 17, 255, 256, 257, 1000, 3333, 6000, 20000]))
+    N = int(rng.choice([128, 256, 384, 512, 1024]))
+    K = int(rng.choice([128, 256, 384, 640, 1024]))
+    kind = ["uniform", "ragged", "empties"][seed % 3]
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(G, N, K, generator=g) * 0.05).to(torch.bfloat16)
+    dout = torch.randn(rows, N, generator=g).to(torch.bfloat16)
+    cum = _counts(kind, G, rows, seed=seed)
+    assert int(cum[-1]) == rows
+    xd = x.to(cuda).requires_grad_(True)
+    wd = w.to(cuda).requires_grad_(True)
+    out = GroupedGemmFunction.apply(xd, wd, cum, int((cum[1:] - cum[:-1]).max()), False)
+    out.backward(dout.to(cuda))
+    ref = _ref_fwd(x, w, cum)
+    dx_ref = torch.zeros(rows, K); dw_ref = torch.zeros(G, N, K)
+    for e in range(G):
+        s, t = int(cum[e]), int(cum[e + 1])
+        dx_ref[s:t] = dout[s:t].float() @ w[e].float()
+        dw_ref[e] = dout[s:t].float().t() @ x[s:t].float()
+    tag = (G, rows, N, K, kind)
+    assert max_abs(out.float().cpu(), ref) <= 2e-2 * max(1.0, float(ref.abs().max())), tag
+    assert mean_rel(out.float().cpu(), ref) <= 4e-3, tag
+    assert mean_rel(xd.grad.float().cpu(), dx_ref) <= 4e-3, tag
+    assert max_abs(wd.grad.float().cpu(), dw_ref) <= 1e-2 * max(1.0, float(dw_ref.abs().max())), tag
+    if float(dw_ref.abs().mean()) > 0:
+        assert mean_rel(wd.grad.float().cpu(), dw_ref) <= 4e-3, tag
