@@ -243,3 +243,43 @@ def test_grouped_gemm_random_shapes(cuda, seed):
     assert max_abs(wd.grad.float().cpu(), dw_ref) <= 1e-2 * max(1.0, float(dw_ref.abs().max())), tag
     if float(dw_ref.abs().mean()) > 0:
         assert mean_rel(wd.grad.float().cpu(), dw_ref) <= 4e-3, tag
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_gathered_merged_mlp_random_shapes(cuda, seed):
+    """Seeded sweep of the bit-identity between the GEMMs that read tokens through input_indices and
+    gather-then-GEMM, over token counts, top-k, expert windows and sizes."""
+    from optimus.models.common.moe import (GatheredMergedMLPFunction, MergedMLPFunction,
+                                           PrepareInputForGroupGemmFunction, build_token_permutation)
+    from util import routed_experts
+    rng = np.random.RandomState(99 + seed)
+    N = int(rng.choice([4, 8, 16, 64]))
+    K = int(rng.choice([1, 2, min(4, N)]))
+    T = int(rng.choice([5, 64, 300, 1024, 5000]))
+    H = int(rng.choice([128, 256, 384, 512]))
+    I = int(rng.choice([128, 256, 384]))
+    start = int(rng.choice([0, N // 4]))
+    end = int(rng.choice([N, max(start + 1, N - N // 4)]))
+    G = end - start
+    g = torch.Generator().manual_seed(seed)
+    se = routed_experts(T, N, K, seed=seed, skew=float(rng.choice([0.0, 1.0]))).to(cuda)
+    cum, cum_ep, ii, oi, _ = build_token_permutation(se, start, end)
+    rows = int(cum[-1].item())
+    ii, oi = ii[:rows], oi[:rows]
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ws = [(torch.randn(G, I, H, generator=g) * 0.05).to(torch.bfloat16),
+          (torch.randn(G, I, H, generator=g) * 0.05).to(torch.bfloat16),
+          (torch.randn(G, H, I, generator=g) * 0.05).to(torch.bfloat16)]
+    dy = torch.randn(rows, H, generator=g).to(torch.bfloat16).to(cuda)
+    results = []
+    for gathered in (False, True):
+        xd = x.to(cuda).requires_grad_(True)
+        wd = [w.to(cuda).requires_grad_(True) for w in ws]
+        if gathered:
+            y = GatheredMergedMLPFunction.apply(xd, ii, cum_ep, oi, *wd, cum)
+        else:
+            y = MergedMLPFunction.apply(PrepareInputForGroupGemmFunction.apply(xd, ii, cum_ep, oi), *wd, cum)
+        y.backward(dy)
+        results.append([y.detach(), xd.grad] + [w.grad for w in wd])
+    for name, a, b in zip(("y", "dx", "dw_gate", "dw_up", "dw_down"), *results):
+        assert torch.equal(a, b), (name, T, K, N, start, end, I, H)
