@@ -90,3 +90,30 @@ def test_reference_shaped_index_ops(cuda, oracle_lib, T, N, K, start, end):
     assert np.array_equal(ii.cpu().numpy(), ref["input_indices"])
     assert np.array_equal(oi.cpu().numpy(), ref["output_indices"])
     assert np.array_equal(si.cpu().numpy(), ref["selected_experts_indices"])
+
+
+@pytest.mark.parametrize("seed", list(range(16)))
+def test_moe_sort_random_shapes(cuda, oracle_lib, seed):
+    """Seeded sweep over token counts (one to a few hundred count blocks), expert counts up to the
+    kernel's limit, top-k and expert windows, bit-exact against the restatement of the reference's
+    K1 -> cumsum -> K3."""
+    rng = np.random.RandomState(7 + seed)
+    N = int(rng.choice([2, 8, 60, 64, 65, 128, 256, 700, 1024]))
+    K = int(rng.choice([1, 2, min(8, N)]))
+    T = int(rng.choice([1, 9, 255, 257, 4096, 30000, 70000]))
+    start = int(rng.choice([0, N // 3]))
+    end = int(rng.choice([N, max(start + 1, N - N // 5)]))
+    dt = [torch.int64, torch.int32][seed % 2]
+    se = routed_experts(T, N, K, seed=seed, skew=float(rng.choice([0.0, 0.8, 2.5])))
+    # the restatement keeps the reference's tokens-per-thread blocking (T a multiple of it); its
+    # result does not depend on the blocking (tests/test_oracle_moe.py), so 1 serves any T
+    ref = oracle_lib.index_construction(se.numpy(), end - start, start, end,
+                                        tokens_per_thread=8 if T % 8 == 0 else 1)
+    cum, cum_ep, ii, oi, si = _gpu_sort(se.to(dt), start, end, cuda)
+    TR = ref["num_routed_tokens"]
+    tag = (T, N, K, start, end)
+    assert np.array_equal(cum, ref["cum_token_counts"]), tag
+    assert np.array_equal(cum_ep, ref["cum_expert_counts_ep"]), tag
+    assert np.array_equal(ii[:TR], ref["input_indices"]), tag
+    assert np.array_equal(oi[:TR], ref["output_indices"]), tag
+    assert np.array_equal(si[:TR], ref["selected_experts_indices"]), tag
