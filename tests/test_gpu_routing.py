@@ -45,6 +45,42 @@ def test_softmax_topk_forward(cuda, T, N, K, renorm, ldt, wdt):
         assert float(((w.cpu() - w_ref).abs() / w_ref).max()) <= 2e-6
 
 
+@pytest.mark.parametrize("seed", list(range(16)))
+def test_softmax_topk_random_shapes(cuda, seed):
+    """Seeded sweep over expert counts (one to eight experts per lane), top-k up to 64, odd token
+    counts, logit scales (sharp and flat distributions), both weight dtypes."""
+    from optimus.models.common.moe import SoftmaxTopkRouterFunction as F
+    rng = np.random.RandomState(31 + seed)
+    N = int(rng.choice([2, 3, 8, 60, 64, 65, 128, 200, 256, 512]))
+    K = int(rng.choice([1, 2, min(8, N), min(64, N)]))
+    T = int(rng.choice([1, 7, 100, 1023, 5000]))
+    renorm = bool(seed % 2)
+    wdt = [torch.float32, torch.bfloat16][(seed // 2) % 2]
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(T, N, generator=g) * float(rng.choice([0.3, 1.0, 4.0]))
+    # rows whose top-(K+1) probabilities are more than 4 ulp apart: there a last-ulp difference in
+    # exp() cannot change the choice, and the result must be the restatement's
+    probs = torch.softmax(logits, 1)
+    top = torch.sort(probs, dim=1, descending=True).values[:, :min(K + 1, N)]
+    ok = ((top[:, :-1] - top[:, 1:]) > 4 * top[:, :-1] * 2.0 ** -23).all(dim=1) if N > 1 else torch.ones(T, dtype=torch.bool)
+    w_ref, e_ref, _ = R.olmoe_router(logits, K, renorm, wdt)
+    w, e = F.apply(logits.to(cuda), K, renorm, wdt)
+    tag = (T, N, K, renorm, wdt)
+    assert int(ok.sum()) >= T // 2, tag
+    assert torch.equal(e.cpu()[ok], e_ref[ok]), tag
+    if wdt == torch.bfloat16:
+        a = w.cpu()[ok].view(torch.int16).int(); b = w_ref[ok].view(torch.int16).int()
+        assert int((a - b).abs().max()) <= 1, tag
+    else:
+        assert float(((w.cpu()[ok] - w_ref[ok]).abs() / w_ref[ok].clamp_min(1e-30)).max()) <= 4e-6, tag
+    # every row, tie or not: K distinct experts, none of them worse than an unselected one
+    sel = probs.gather(1, e.cpu())
+    rest = probs.scatter(1, e.cpu(), -1.0)
+    assert bool((sel.min(1).values >= rest.max(1).values * (1 - 1e-6)).all()), tag
+    srt = torch.sort(e.cpu(), 1).values
+    assert bool((srt[:, 1:] != srt[:, :-1]).all()), tag
+
+
 def test_softmax_topk_bf16_logits_and_ties(cuda):
     """bf16 logits tie often; the rule is (probability desc, expert index asc) = stable sort."""
     from optimus.models.common.moe import SoftmaxTopkRouterFunction as F
