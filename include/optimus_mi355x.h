@@ -131,6 +131,16 @@ int om_router_gate_softmax_topk(const void *x, const void *gate_weight, int64_t 
 int om_router_gate_logits(const void *x, const void *gate_weight, int64_t T, int H, int N,
                           float *logits_out, void *stream);
 
+/* om_router_gate_logits_split: the same projection as om_router_gate_logits for gates with many
+ * experts (the DeepSeek-V3 router, 256 x 7168): 128 tokens and a slice of H per block, the weight
+ * tile shared through LDS, the slices added in a fixed order.  N <= 256, H a multiple of 64.
+ * workspace: om_router_gate_logits_split_workspace_bytes(T,H,N) bytes, 16-byte aligned
+ * (negative = error code).  Same value as om_router_gate_logits up to the order of the sum.   */
+int64_t om_router_gate_logits_split_workspace_bytes(int64_t T, int H, int N);
+int om_router_gate_logits_split(const void *x, const void *gate_weight, int64_t T, int H, int N,
+                                float *logits_out, void *workspace, int64_t workspace_bytes,
+                                void *stream);
+
 /* om_router_gate_wgrad: gradient of the gate's weight,
  *   dweight[n,h] = sum_t dlogits[t,n] * x[t,h]
  * i.e. what autograd computes for the nn.Linear behind `router_logits = self.gate(hidden_states)`

@@ -40,6 +40,9 @@ SIGNATURES = {
     "om_router_gate_softmax_topk": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_int, c_int,
                                             c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
     "om_router_gate_logits": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p, c_void_p]),
+    "om_router_gate_logits_split_workspace_bytes": (c_i64, [c_i64, c_int, c_int]),
+    "om_router_gate_logits_split": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p, c_void_p,
+                                            c_i64, c_void_p]),
     "om_router_gate_wgrad_workspace_bytes": (c_i64, [c_i64, c_int, c_int]),
     "om_router_gate_wgrad": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p, c_int, c_void_p,
                                      c_i64, c_void_p]),
@@ -112,7 +115,7 @@ launch_log = None
 launch_filter = None   # optional set of entry-point names: only these are timed while launch_log is set
 _UNTIMED = {"om_version", "om_arch", "om_strerror", "om_moe_sort_workspace_bytes",
             "om_router_balance_workspace_bytes", "om_rmsnorm_bwd_workspace_bytes",
-            "om_router_gate_wgrad_workspace_bytes"}
+            "om_router_gate_wgrad_workspace_bytes", "om_router_gate_logits_split_workspace_bytes"}
 
 
 class NativeLibraryError(RuntimeError):

@@ -107,6 +107,17 @@ def gate_kernel_fits(x, weight):
     return H % (512 if N <= 64 else 256 if N <= 128 else 64) == 0
 
 
+def gate_logits_kernel_fits(x, weight):
+    """Shapes and dtypes GateLogitsFunction takes: om_router_gate_logits up to 64 experts,
+    om_router_gate_logits_split above."""
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
+        return False
+    N, H = weight.shape
+    if N > 256 or x.shape[0] == 0:
+        return False
+    return H % (512 if N <= 64 else 64) == 0
+
+
 def gate_wgrad_kernel_fits(x, weight):
     """Shapes om_router_gate_wgrad takes."""
     N, H = weight.shape
@@ -155,8 +166,19 @@ class GateLogitsFunction(torch.autograd.Function):
     def forward(ctx, x, weight):
         T, (N, H) = x.shape[0], weight.shape
         logits = torch.empty((T, N), dtype=torch.float32, device=x.device)
-        _n.check(_n.lib().om_router_gate_logits(_n.ptr(x), _n.ptr(weight), T, H, N, _n.ptr(logits),
-                                                _n.stream()), "om_router_gate_logits")
+        lib = _n.lib()
+        if N > 64 and H % 64 == 0:
+            # many experts: the weight no longer fits a block's re-reads; split over H instead
+            ws_bytes = lib.om_router_gate_logits_split_workspace_bytes(T, H, N)
+            if ws_bytes < 0:
+                _n.check(int(ws_bytes), "om_router_gate_logits_split_workspace_bytes")
+            workspace = torch.empty(max(int(ws_bytes), 16), dtype=torch.uint8, device=x.device)
+            _n.check(lib.om_router_gate_logits_split(_n.ptr(x), _n.ptr(weight), T, H, N, _n.ptr(logits),
+                                                     _n.ptr(workspace), int(ws_bytes), _n.stream()),
+                     "om_router_gate_logits_split")
+        else:
+            _n.check(lib.om_router_gate_logits(_n.ptr(x), _n.ptr(weight), T, H, N, _n.ptr(logits),
+                                               _n.stream()), "om_router_gate_logits")
         ctx.save_for_backward(x, weight)
         return logits
 
@@ -168,7 +190,7 @@ class GateLogitsFunction(torch.autograd.Function):
 
 def fp32_logits(x, weight):
     """Router logits in float32 from 2-D x [T,H] and weight [N,H] (the gate's nn.Linear weight)."""
-    if gate_kernel_fits(x, weight):
+    if gate_logits_kernel_fits(x, weight):
         return GateLogitsFunction.apply(x.contiguous(), weight.contiguous())
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda:
         return Fp32LogitsFunction.apply(x.contiguous(), weight.contiguous())

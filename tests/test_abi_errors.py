@@ -61,6 +61,14 @@ def test_routers(lib):
     assert lib.om_router_gate_softmax_topk(ODD, P, 8, 2048, 64, 8, 0, P, P, BF16, P, None) == ALIGN
     assert lib.om_router_gate_softmax_topk(P, P, 8, 2048, 64, 8, 0, P, None, BF16, P, None) == NULL
     assert lib.om_router_gate_logits(P, P, 8, 2048, 64, None, None) == NULL
+    need = lib.om_router_gate_logits_split_workspace_bytes(8192, 7168, 256)
+    assert need > 0 and need % 16 == 0
+    assert lib.om_router_gate_logits_split_workspace_bytes(8192, 7100, 256) == SHAPE     # H % 64
+    assert lib.om_router_gate_logits_split_workspace_bytes(8192, 7168, 300) == SHAPE     # N > 256
+    assert lib.om_router_gate_logits_split(P, P, 8192, 7168, 256, P, P, need - 1, None) == WORKSPACE
+    assert lib.om_router_gate_logits_split(P, None, 8192, 7168, 256, P, P, need, None) == NULL
+    assert lib.om_router_gate_logits_split(ODD, P, 8192, 7168, 256, P, P, need, None) == ALIGN
+    assert lib.om_router_gate_logits_split(P, P, 0, 7168, 256, P, P, 0, None) == OK
     need = lib.om_router_gate_wgrad_workspace_bytes(16384, 2048, 64)
     assert need > 0 and need % 16 == 0
     assert lib.om_router_gate_wgrad_workspace_bytes(16384, 2000, 64) == SHAPE      # H % 128

@@ -180,13 +180,17 @@ def _gate_inputs(T, H, N, seed):
 
 
 @pytest.mark.parametrize("T,H,N", [(1000, 2048, 64), (64, 512, 8), (33, 1024, 128), (300, 7168, 256),
-                                   (4096, 2048, 60)])
+                                   (4096, 2048, 60),
+                                   # more than 64 experts: the kernel that shares the weight tile
+                                   # through LDS and splits H (odd step counts, padded expert rows,
+                                   # a partial last 128-token block, one and several slices)
+                                   (8192, 7168, 256), (1000, 1024, 130), (129, 320, 96), (5, 64, 200)])
 def test_gate_logits_match_fp32_matmul(cuda, T, H, N):
     """fp32 logits from bf16 operands: the products are exact, only the order of the fp32 sum differs
     from the CPU matmul of the up-cast operands."""
-    from optimus.models.common.moe import fp32_logits, gate_kernel_fits
+    from optimus.models.common.moe import fp32_logits, gate_logits_kernel_fits
     x, w = _gate_inputs(T, H, N, seed=T + N)
-    assert gate_kernel_fits(x.to(cuda), w.to(cuda))
+    assert gate_logits_kernel_fits(x.to(cuda), w.to(cuda))
     got = fp32_logits(x.to(cuda), w.to(cuda)).cpu()
     ref = x.float() @ w.float().t()
     exact = (x.double() @ w.double().t())
