@@ -45,6 +45,8 @@ MEASURED_TRAFFIC_BYTES = {
 GEMM_ENTRY_PRODUCTS = {     # C-ABI entry -> number of [rows x N x K] products per launch
     "om_merged_mlp_gate_up_fwd": 2, "om_grouped_gemm_fwd": 1, "om_grouped_gemm_wgrad": 1,
     "om_merged_mlp_gate_up_fwd_gathered": 2, "om_grouped_gemm_wgrad_gathered": 1,
+    "om_merged_mlp_gate_up_fwd_weighted": 2, "om_grouped_gemm_wgrad_gathered_out": 1,
+    "om_merged_mlp_down_dgrad_weighted": 1,
     "om_merged_mlp_down_dgrad": 1, "om_merged_mlp_gate_up_dgrad": 2, "om_grouped_gemm_dgrad": 1,
 }
 

@@ -379,6 +379,57 @@ int om_grouped_gemm_wgrad_gathered(const void *output_grad, const void *input,
                                    const int32_t *cum_token_counts, int64_t rows, int G, int N,
                                    int K, int64_t w_stride, void *stream);
 
+/* The combine's routing weight folded into the expert MLP.  The reference multiplies by w[t,k]
+ * when it sums the experts' outputs (GroupGemmOutputReductionFunction, optimus/models/common/
+ * moe.py:284-377) and its reduce_ggemm_output kernel already has a skip_weights_scaling switch
+ * for rows that arrive scaled (sparse_moe_block.sycl:292-303).  Since the down projection is linear,
+ *   w * ((silu(g) * u) @ Wd.T) = ((w * silu(g) * u) @ Wd.T),
+ * the weight can be applied where h is formed, and in the backward pass the [rows, H] gradient of
+ * the experts' output, w[t,k] * dfinal[t,:], never has to be written: the down projection's two
+ * backward GEMMs read dfinal through input_indices, and the SwiGLU-backward epilogue applies w and
+ * forms the routing weights' gradient.  Same mathematics as the reference's sequence; the bf16
+ * roundings fall in different places (h is rounded after the weight, not before), so results agree
+ * with the two-step form to bf16 accuracy, not bit for bit.
+ *   om_moe_row_weights       : row_weights[pos] = w[t,k] for every routed entry rt (pos =
+ *                              output_indices[rt], t = input_indices[pos], k = sel_idx[rt]); fp32 [RT]
+ *   om_merged_mlp_gate_up_fwd_weighted : as ..._gate_up_fwd_gathered, h = bf16(row_weights[r] *
+ *                              silu(g) * u) (g and u are stored unweighted)
+ *   om_sum_ggemm_output      : final[t,:] = (residual[t,:] +) bf16(sum of the token's rows), no weights;
+ *                              residual may be null
+ *   om_grouped_gemm_wgrad_gathered_out : as om_grouped_gemm_wgrad with output_grad = dfinal
+ *                              [src_rows, N] read through output_grad_rows = input_indices [rows]
+ *   om_merged_mlp_down_dgrad_weighted  : dh' = dfinal[dy_rows[r]] @ Wd[e];
+ *                              row_dot[part][r] = sum over the part's 64 columns of dh' * silu(g) * u
+ *                              (parts = om_merged_mlp_row_dot_parts(I) = I / 64, fp32 [parts, rows]);
+ *                              then as om_merged_mlp_down_dgrad with dh = row_weights[r] * dh'
+ *   om_moe_row_weights_grad  : dw[t,k] = sum over parts (in order) of row_dot[part][pos]; entries of
+ *                              pairs outside the expert window are not written (pre-zero them)   */
+int om_moe_row_weights(const void *routing_weights, const int32_t *selected_experts_indices,
+                       const int32_t *input_indices, const int32_t *output_indices,
+                       float *row_weights, int64_t RT, int K, int weights_dtype, void *stream);
+int om_merged_mlp_gate_up_fwd_weighted(const void *x, const int32_t *x_rows, int64_t src_rows,
+                                       const void *w_gate, const void *w_up, const float *row_weights,
+                                       void *g, void *u, void *h, const int32_t *cum_token_counts,
+                                       int64_t rows, int G, int I, int H, int64_t w_stride,
+                                       void *stream);
+int om_sum_ggemm_output(const void *ggemm_output, const int32_t *cum_expert_counts_ep,
+                        const int32_t *output_indices, const void *residual,
+                        void *final_hidden_states, int64_t T, int64_t E, int dtype, void *stream);
+int om_grouped_gemm_wgrad_gathered_out(const void *output_grad, const int32_t *output_grad_rows,
+                                       int64_t src_rows, const void *input, void *weight_grad,
+                                       const int32_t *cum_token_counts, int64_t rows, int G, int N,
+                                       int K, int64_t w_stride, void *stream);
+int om_merged_mlp_row_dot_parts(int I);
+int om_merged_mlp_down_dgrad_weighted(const void *dy, const int32_t *dy_rows, int64_t src_rows,
+                                      const void *w_down, const void *g, const void *u,
+                                      const float *row_weights, void *dg, void *du, float *row_dot,
+                                      const int32_t *cum_token_counts, int64_t rows, int G, int I,
+                                      int H, int64_t w_stride, void *stream);
+int om_moe_row_weights_grad(const float *row_dot, int parts, const int32_t *selected_experts_indices,
+                            const int32_t *input_indices, const int32_t *output_indices,
+                            void *routing_weights_grad, int64_t RT, int K, int weights_dtype,
+                            void *stream);
+
 /* Stand-alone SwiGLU glue (moe.py:401-402 forward; moe.py:37-41 and :133-147 backward),
  * for callers that keep the three GEMMs separate.  n elements, dtype OM_F32 or OM_BF16.   */
 int om_swiglu_fwd(const void *g, const void *u, void *h, int64_t n, int dtype, void *stream);

@@ -33,7 +33,12 @@ namespace {
 enum { CONTIG = 0, STRIDED = 1 };
 // An operand's rows can be taken through an index instead of in order: the token gather that
 // precedes the expert GEMMs (ggemm_input = hidden_states[input_indices]) folded into the loads.
-enum { GATHER_NONE = 0, GATHER_A = 1 /* fwd: A rows */, GATHER_B = 2 /* wgrad: contraction rows of B */ };
+enum {
+    GATHER_NONE = 0,
+    GATHER_A = 1,    // fwd/dgrad: A rows
+    GATHER_B = 2,    // wgrad: contraction rows of B
+    GATHER_WA = 3    // wgrad: contraction rows of A
+};
 enum {
     EPI_STORE = 0,        // C = acc
     EPI_SWIGLU = 1,       // even 32-col accumulators = gate, odd = up: store g, u, h
@@ -64,7 +69,10 @@ struct GemmParams {
     const uint16_t *G;   // EPI_SWIGLU_BWD: saved g
     const uint16_t *U;   // EPI_SWIGLU_BWD: saved u
     const int32_t *cum;  // [G+1] device
-    const int32_t *row_index;   // GATHER_A: A row of sorted row r; GATHER_B: B row of contraction row c
+    const int32_t *row_index;   // GATHER_A: A row of sorted row r; GATHER_B / GATHER_WA: B / A row of contraction row c
+    // ROWW kernels (the routing weight folded into the expert MLP):
+    const float *row_scale;     // [rows] weight of each sorted row
+    float *row_dot;             // EPI_SWIGLU_BWD: [n_cols / COLS][rows] partial sums of dh * silu(g) * u
     int64_t lda, ldb, ldc;      // leading dimensions, elements
     int64_t strideB, strideC;   // per-expert strides, elements
     int64_t rows;               // allocated activation rows (upper bound of cum[G])
@@ -138,6 +146,20 @@ __device__ __forceinline__ float fast_sigmoid(float x) {
     return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
 }
 
+// Sum over aligned groups of N neighbouring lanes (N = 4, 8 or 16); every lane of the group gets
+// it.  DPP: swap within pairs, swap pairs within quads, mirror within 8, mirror within 16.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+template <int N> __device__ __forceinline__ float lane_group_sum(float v) {
+    static_assert(N == 4 || N == 8 || N == 16, "group size");
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    if (N >= 8) v += dpp_move<0x141>(v);
+    if (N >= 16) v += dpp_move<0x140>(v);
+    return v;
+}
+
 __device__ __forceinline__ void unpack4_bf16(u32x2 v, float *f) {
     f[0] = __uint_as_float(v[0] << 16);
     f[1] = __uint_as_float(v[0] & 0xffff0000u);
@@ -190,10 +212,13 @@ __device__ __forceinline__ bool find_tile(const int *tile_end, const int *seg, i
     return false;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE,
+          bool ROWW = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const GemmParams p) {
     static_assert(GATHER == GATHER_NONE || (GATHER == GATHER_A && AKIND == CONTIG && EPI != EPI_WGRAD) ||
-                      (GATHER == GATHER_B && BKIND == STRIDED && EPI == EPI_WGRAD), "gather variants");
+                      (GATHER == GATHER_B && BKIND == STRIDED && EPI == EPI_WGRAD) ||
+                      (GATHER == GATHER_WA && AKIND == STRIDED && EPI == EPI_WGRAD), "gather variants");
+    static_assert(!ROWW || EPI == EPI_SWIGLU || EPI == EPI_SWIGLU_BWD, "row weights belong to the SwiGLU epilogues");
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
     constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 accumulators per wavefront
@@ -237,6 +262,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     int b_crow[B_LOADS];
     bool b_up[B_LOADS];   // EPI_SWIGLU: this LDS row comes from the up matrix
     int b_src[GATHER == GATHER_B ? B_LOADS : 1];   // GATHER_B: source rows of the next B loads
+    int a_src[GATHER == GATHER_WA ? A_LOADS : 1];  // GATHER_WA: source rows of the next A loads
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
         constexpr int CPR = BM / 8;
@@ -263,6 +289,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         for (int i = 0; i < B_LOADS; i++) {
             const int c = min(c0 + b_crow[i], c_len - 1);   // past the segment: any valid row (A is zeroed)
             b_src[GATHER == GATHER_B ? i : 0] = p.row_index[c_begin + c];
+        }
+    };
+
+    auto load_a_src = [&](int step) {   // GATHER_WA: the same for the A rows
+        if (GATHER != GATHER_WA || step >= loop_steps) return;
+        const int c0 = (step < steps_per_phase ? rotated(step) : step) * BK;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; i++) {
+            const int c = min(c0 + a_crow[i], c_len - 1);   // past the segment: any valid row (zeroed in LDS)
+            a_src[GATHER == GATHER_WA ? i : 0] = p.row_index[c_begin + c];
         }
     };
 
@@ -349,6 +385,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             }
         }
         load_b_src(0);
+        load_a_src(0);
         return true;
     };
 
@@ -377,10 +414,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             } else {
                 int c = c0 + a_crow[i];
                 if (EPI == EPI_WGRAD) c = min(c, c_len - 1);  // stay in the segment; zeroed below
-                off = static_cast<uint32_t>(a_off[i] + (c_begin + c) * lda32) * 2u;
+                if (GATHER == GATHER_WA)
+                    off = static_cast<uint32_t>(a_off[i] + a_src[GATHER == GATHER_WA ? i : 0] * lda32) * 2u;
+                else
+                    off = static_cast<uint32_t>(a_off[i] + (c_begin + c) * lda32) * 2u;
             }
             load16_to_lds(Ap + off, sa + i * 1024);
         }
+        if (hi >= A_LOADS && lo < A_LOADS) load_a_src(step + 1);   // this step's A loads are out
 #pragma unroll
         for (int i = 0; i < B_LOADS; i++) {
             if (A_LOADS + i < lo || A_LOADS + i >= hi) continue;
@@ -646,10 +687,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     };
     const int col0 = (EPI == EPI_SWIGLU) ? e_n0 + (wn_e * WN) / 2 : e_n0 + wn_e * WN;   // first output column
     uint16_t *Cb = p.C + (EPI == EPI_WGRAD ? e_expert * p.strideC : 0);
+    // ROWW forward: the weights of this lane's row in every strip, fetched together up front
+    float wrow_all[(ROWW && EPI == EPI_SWIGLU) ? TM : 1];
+    if (ROWW && EPI == EPI_SWIGLU) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int64_t m = static_cast<int64_t>(e_row_begin) + wm_e * WM + i * 32 + lrow;
+            wrow_all[(ROWW && EPI == EPI_SWIGLU) ? i : 0] = (m < e_row_end) ? p.row_scale[m] : 0.0f;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int64_t m0 = static_cast<int64_t>(e_row_begin) + wm_e * WM + i * 32;  // first row of the strip
         if (EPI == EPI_SWIGLU) {
+            const float wrow = wrow_all[(ROWW && EPI == EPI_SWIGLU) ? i : 0];   // ROWW: h = w[row] * silu(g) * u, one rounding
 #pragma unroll
             for (int j = 0; j < TN; j += 2)
 #pragma unroll
@@ -659,6 +710,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                     for (int x = 0; x < 4; x++) {
                         const float gv = acc[i][j][rq * 4 + x], uv = acc[i][j + 1][rq * 4 + x];
                         hv[x] = (gv * fast_sigmoid(gv)) * uv;
+                        if (ROWW) hv[x] *= wrow;
                     }
                     const int col = (j / 2) * 32 + rq * 8 + lcol;
                     strip_put(0, col, acc[i][j][rq * 4], acc[i][j][rq * 4 + 1], acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3]);
@@ -676,6 +728,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         strip_sync();
         if (EPI == EPI_SWIGLU_BWD) {
             u32x4 gq[ITS], uq[ITS];
+            // ROWW: lane l fetches the weight of strip row l % 32 along with the g/u loads; the
+            // lanes that work on a row pick it up with a lane read
+            float w_strip = 0.0f;
+            if (ROWW && m0 + (lane_e & 31) < e_row_end) w_strip = p.row_scale[m0 + (lane_e & 31)];
 #pragma unroll
             for (int it = 0; it < ITS; it++) {
                 const int q = it * 64 + lane_e;
@@ -690,6 +746,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             for (int it = 0; it < ITS; it++) {
                 const int q = it * 64 + lane_e;
                 const int64_t m = m0 + q / CPRW;
+                float dot = 0.0f;   // ROWW: this lane's part of sum_i dh[m][i] * silu(g[m][i]) * u[m][i]
+                const float wr = ROWW ? __shfl(w_strip, q / CPRW, 64) : 1.0f;
                 if (m < e_row_end) {
                     float dh[8], gv[8], uv[8], dg[8], du[8];
                     Elem<uint16_t>::unpack(strip_get(0, q / CPRW, q % CPRW), dh);
@@ -698,7 +756,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 #pragma unroll
                     for (int x = 0; x < 8; x++) {
                         const float sg = fast_sigmoid(gv[x]);
-                        du[x] = dh[x] * (gv[x] * sg);
+                        const float sl = gv[x] * sg;
+                        if (ROWW) {
+                            // acc is the gradient of w * silu(g) * u: the routing weight's gradient
+                            // is its product with silu(g) * u, the activation's gets the factor w
+                            dot += dh[x] * (sl * uv[x]);
+                            dh[x] *= wr;
+                        }
+                        du[x] = dh[x] * sl;
                         dg[x] = (dh[x] * uv[x]) * (sg * (1.0f + gv[x] * (1.0f - sg)));
                     }
                     const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
@@ -710,6 +775,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                     }
                     *reinterpret_cast<u32x4 *>(p.C + o) = vg;
                     *reinterpret_cast<u32x4 *>(p.C1 + o) = vu;
+                }
+                if (ROWW) {
+                    // the CPRW lanes of a row are neighbours: add them up in a fixed order and let
+                    // the first one store the sum for this wavefront's column range
+                    dot = lane_group_sum<CPRW>(dot);
+                    if (q % CPRW == 0 && m < e_row_end) p.row_dot[(col0 / COLS) * p.rows + m] = dot;
                 }
             }
         } else {
@@ -765,7 +836,7 @@ template <int BM> struct Waves {
     static constexpr int N = (BM == 256) ? OM_WAVES_N : 2;
 };
 
-template <int BM, int BN, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE>
+template <int BM, int BN, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = false>
 int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad family
     constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
     if (p.n_experts > MAX_EXPERTS) return OM_ERR_SHAPE;   // the tile table lives in LDS
@@ -773,19 +844,24 @@ int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad f
     const int64_t tiles = static_cast<int64_t>(p.m_tiles_max) * (p.n_cols / BN_OUT);
     if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
     p.total_tiles = static_cast<int>(tiles);
-    ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI, GATHER>
+    ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI, GATHER, ROWW>
         <<<dim3(persistent_blocks<BM>(tiles)), dim3(Waves<BM>::M * Waves<BM>::N * 64), 0, st>>>(p);
     return om_launch_status();
 }
 
-template <int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE>
+// the tile shape launch_rows_auto picks
+template <int EPI> bool uses_big_tile(int n_cols, int n_experts, int64_t rows) {
+    constexpr int div = (EPI == EPI_SWIGLU) ? 2 : 1;
+    return n_cols % (256 / div) == 0 && rows >= static_cast<int64_t>(n_experts) * 192;
+}
+
+template <int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = false>
 int launch_rows_auto(GemmParams &p, int64_t rows, hipStream_t st) {
     constexpr int div = (EPI == EPI_SWIGLU) ? 2 : 1;
-    const bool big_ok = p.n_cols % (256 / div) == 0;
-    const bool few_rows = rows < static_cast<int64_t>(p.n_experts) * 192;
-    if (big_ok && !few_rows) return launch_rows<256, 256, AKIND, BKIND, EPI, GATHER>(p, rows, st);
+    if (uses_big_tile<EPI>(p.n_cols, p.n_experts, rows))
+        return launch_rows<256, 256, AKIND, BKIND, EPI, GATHER, ROWW>(p, rows, st);
     if (p.n_cols % (128 / div) != 0) return OM_ERR_SHAPE;
-    return launch_rows<128, 128, AKIND, BKIND, EPI, GATHER>(p, rows, st);
+    return launch_rows<128, 128, AKIND, BKIND, EPI, GATHER, ROWW>(p, rows, st);
 }
 
 }  // namespace
@@ -829,11 +905,12 @@ extern "C" int om_grouped_gemm_dgrad(const void *output_grad, const void *weight
 }
 
 namespace {
-// weight gradient; `input_rows` != null: contraction row c of `input` is row input_rows[c] of a
-// [src_rows, K] matrix (the token gather folded into the loads)
-int wgrad_launch(const void *output_grad, const void *input, const int32_t *input_rows, int64_t src_rows,
-                 void *weight_grad, const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
-                 int64_t w_stride, void *stream) {
+// weight gradient; gather == GATHER_B: contraction row c of `input` is row index[c] of a
+// [src_rows, K] matrix; gather == GATHER_WA: contraction row c of `output_grad` is row index[c] of a
+// [src_rows, N] matrix (the token gather folded into the loads)
+int wgrad_launch(const void *output_grad, const void *input, const int32_t *index, int gather,
+                 int64_t src_rows, void *weight_grad, const int32_t *cum_token_counts, int64_t rows, int G,
+                 int N, int K, int64_t w_stride, void *stream) {
     if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
     // rows == 0 (nothing routed to these experts): the activations may be empty tensors without
     // storage; the launch then only writes zeros
@@ -844,10 +921,11 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inpu
     p.B[0] = static_cast<const uint16_t *>(input);        // [rows, K] (or [src_rows, K] through input_rows)
     p.C = static_cast<uint16_t *>(weight_grad);           // [G, N, K]
     p.cum = cum_token_counts;
-    p.row_index = input_rows;
+    p.row_index = index;
     p.lda = N; p.ldb = K; p.ldc = K;
     p.strideC = w_stride ? w_stride : static_cast<int64_t>(N) * K;
-    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideC * G) || !fits31(src_rows * K))
+    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideC * G) ||
+        !fits31(src_rows * (gather == GATHER_WA ? N : K)))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
     hipStream_t st = om_stream(stream);
@@ -858,14 +936,18 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inpu
     p.total_tiles = static_cast<int>(tiles);
     const dim3 grid_big(persistent_blocks<256>(tiles)), block_big(Waves<256>::M * Waves<256>::N * 64);
     const dim3 grid_small(persistent_blocks<128>(tiles)), block_small(256);
-    if (big && !input_rows)
+    if (big && gather == GATHER_NONE)
         ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD><<<grid_big, block_big, 0, st>>>(p);
-    else if (big)
+    else if (big && gather == GATHER_B)
         ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD, GATHER_B><<<grid_big, block_big, 0, st>>>(p);
-    else if (!input_rows)
+    else if (big)
+        ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD, GATHER_WA><<<grid_big, block_big, 0, st>>>(p);
+    else if (gather == GATHER_NONE)
         ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD><<<grid_small, block_small, 0, st>>>(p);
-    else
+    else if (gather == GATHER_B)
         ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD, GATHER_B><<<grid_small, block_small, 0, st>>>(p);
+    else
+        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD, GATHER_WA><<<grid_small, block_small, 0, st>>>(p);
     return om_launch_status();
 }
 }  // namespace
@@ -873,8 +955,8 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inpu
 extern "C" int om_grouped_gemm_wgrad(const void *output_grad, const void *input, void *weight_grad,
                                      const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                      int64_t w_stride, void *stream) {
-    return wgrad_launch(output_grad, input, nullptr, 0, weight_grad, cum_token_counts, rows, G, N, K,
-                        w_stride, stream);
+    return wgrad_launch(output_grad, input, nullptr, GATHER_NONE, 0, weight_grad, cum_token_counts, rows, G,
+                        N, K, w_stride, stream);
 }
 
 extern "C" int om_grouped_gemm_wgrad_gathered(const void *output_grad, const void *input,
@@ -884,15 +966,27 @@ extern "C" int om_grouped_gemm_wgrad_gathered(const void *output_grad, const voi
                                               void *stream) {
     if (!input_rows) return OM_ERR_NULL;
     if (src_rows < 1) return OM_ERR_SHAPE;
-    return wgrad_launch(output_grad, input, input_rows, src_rows, weight_grad, cum_token_counts, rows, G,
-                        N, K, w_stride, stream);
+    return wgrad_launch(output_grad, input, input_rows, GATHER_B, src_rows, weight_grad, cum_token_counts,
+                        rows, G, N, K, w_stride, stream);
+}
+
+extern "C" int om_grouped_gemm_wgrad_gathered_out(const void *output_grad, const int32_t *output_grad_rows,
+                                                  int64_t src_rows, const void *input, void *weight_grad,
+                                                  const int32_t *cum_token_counts, int64_t rows, int G,
+                                                  int N, int K, int64_t w_stride, void *stream) {
+    if (!output_grad_rows) return OM_ERR_NULL;
+    if (src_rows < 1) return OM_ERR_SHAPE;
+    return wgrad_launch(output_grad, input, output_grad_rows, GATHER_WA, src_rows, weight_grad,
+                        cum_token_counts, rows, G, N, K, w_stride, stream);
 }
 
 namespace {
 // `x_rows` != null: sorted row r of the activations is row x_rows[r] of x [src_rows, H]
+// `row_weights` != null (needs x_rows): h = row_weights[r] * silu(g) * u
 int gate_up_fwd_launch(const void *x, const int32_t *x_rows, int64_t src_rows, const void *w_gate,
-                       const void *w_up, void *g, void *u, void *h, const int32_t *cum_token_counts,
-                       int64_t rows, int G, int I, int H, int64_t w_stride, void *stream) {
+                       const void *w_up, const float *row_weights, void *g, void *u, void *h,
+                       const int32_t *cum_token_counts, int64_t rows, int G, int I, int H,
+                       int64_t w_stride, void *stream) {
     if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 128)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!x || !w_gate || !w_up || !g || !u || !h || !cum_token_counts) return OM_ERR_NULL;
@@ -908,11 +1002,13 @@ int gate_up_fwd_launch(const void *x, const int32_t *x_rows, int64_t src_rows, c
     p.C2 = static_cast<uint16_t *>(h);
     p.cum = cum_token_counts;
     p.row_index = x_rows;
+    p.row_scale = row_weights;
     p.lda = H; p.ldb = H; p.ldc = I;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(I) * H;
     if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G) || !fits31(src_rows * H))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = I; p.kc = H; p.phases = 1;
+    if (row_weights) return launch_rows_auto<CONTIG, CONTIG, EPI_SWIGLU, GATHER_A, true>(p, rows, om_stream(stream));
     if (x_rows) return launch_rows_auto<CONTIG, CONTIG, EPI_SWIGLU, GATHER_A>(p, rows, om_stream(stream));
     return launch_rows_auto<CONTIG, CONTIG, EPI_SWIGLU>(p, rows, om_stream(stream));
 }
@@ -922,8 +1018,8 @@ extern "C" int om_merged_mlp_gate_up_fwd(const void *x, const void *w_gate, cons
                                          void *u, void *h, const int32_t *cum_token_counts,
                                          int64_t rows, int G, int I, int H, int64_t w_stride,
                                          void *stream) {
-    return gate_up_fwd_launch(x, nullptr, 0, w_gate, w_up, g, u, h, cum_token_counts, rows, G, I, H,
-                              w_stride, stream);
+    return gate_up_fwd_launch(x, nullptr, 0, w_gate, w_up, nullptr, g, u, h, cum_token_counts, rows, G, I,
+                              H, w_stride, stream);
 }
 
 extern "C" int om_merged_mlp_gate_up_fwd_gathered(const void *x, const int32_t *x_rows, int64_t src_rows,
@@ -933,14 +1029,33 @@ extern "C" int om_merged_mlp_gate_up_fwd_gathered(const void *x, const int32_t *
                                                   void *stream) {
     if (rows > 0 && !x_rows) return OM_ERR_NULL;
     if (src_rows < 1 && rows > 0) return OM_ERR_SHAPE;
-    return gate_up_fwd_launch(x, x_rows, src_rows, w_gate, w_up, g, u, h, cum_token_counts, rows, G, I, H,
-                              w_stride, stream);
+    return gate_up_fwd_launch(x, x_rows, src_rows, w_gate, w_up, nullptr, g, u, h, cum_token_counts, rows,
+                              G, I, H, w_stride, stream);
 }
 
-extern "C" int om_merged_mlp_down_dgrad(const void *dy, const void *w_down, const void *g, const void *u,
-                                        void *dg, void *du, const int32_t *cum_token_counts,
-                                        int64_t rows, int G, int I, int H, int64_t w_stride,
-                                        void *stream) {
+extern "C" int om_merged_mlp_gate_up_fwd_weighted(const void *x, const int32_t *x_rows, int64_t src_rows,
+                                                  const void *w_gate, const void *w_up,
+                                                  const float *row_weights, void *g, void *u, void *h,
+                                                  const int32_t *cum_token_counts, int64_t rows, int G,
+                                                  int I, int H, int64_t w_stride, void *stream) {
+    if (rows > 0 && (!x_rows || !row_weights)) return OM_ERR_NULL;
+    if (src_rows < 1 && rows > 0) return OM_ERR_SHAPE;
+    return gate_up_fwd_launch(x, x_rows, src_rows, w_gate, w_up, row_weights, g, u, h, cum_token_counts,
+                              rows, G, I, H, w_stride, stream);
+}
+
+namespace {
+// columns of the intermediate size that one wavefront's epilogue covers (both tile shapes): the
+// granularity of the row_dot partial sums
+constexpr int ROW_DOT_COLS = 64;
+static_assert(256 / Waves<256>::N == ROW_DOT_COLS && 128 / Waves<128>::N == ROW_DOT_COLS, "row_dot layout");
+
+// `dy_rows` != null: sorted row r of dy is row dy_rows[r] of a [src_rows, H] matrix, the result is
+// scaled by row_weights[r] and row_dot receives the partial sums of (dy W) * silu(g) * u
+int down_dgrad_launch(const void *dy, const int32_t *dy_rows, int64_t src_rows, const void *w_down,
+                      const void *g, const void *u, const float *row_weights, void *dg, void *du,
+                      float *row_dot, const int32_t *cum_token_counts, int64_t rows, int G, int I, int H,
+                      int64_t w_stride, void *stream) {
     if (rows < 0 || G < 1 || !mult(I, 128) || !mult(H, 128)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!dy || !w_down || !g || !u || !dg || !du || !cum_token_counts) return OM_ERR_NULL;
@@ -955,11 +1070,42 @@ extern "C" int om_merged_mlp_down_dgrad(const void *dy, const void *w_down, cons
     p.G = static_cast<const uint16_t *>(g);
     p.U = static_cast<const uint16_t *>(u);
     p.cum = cum_token_counts;
+    p.row_index = dy_rows;
+    p.row_scale = row_weights;
+    p.row_dot = row_dot;
     p.lda = H; p.ldb = I; p.ldc = I;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(H) * I;
-    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
+    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G) || !fits31(src_rows * H))
+        return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = I; p.kc = H; p.phases = 1;
+    if (dy_rows) return launch_rows_auto<CONTIG, STRIDED, EPI_SWIGLU_BWD, GATHER_A, true>(p, rows, om_stream(stream));
     return launch_rows_auto<CONTIG, STRIDED, EPI_SWIGLU_BWD>(p, rows, om_stream(stream));
+}
+}  // namespace
+
+extern "C" int om_merged_mlp_down_dgrad(const void *dy, const void *w_down, const void *g, const void *u,
+                                        void *dg, void *du, const int32_t *cum_token_counts,
+                                        int64_t rows, int G, int I, int H, int64_t w_stride,
+                                        void *stream) {
+    return down_dgrad_launch(dy, nullptr, 0, w_down, g, u, nullptr, dg, du, nullptr, cum_token_counts, rows,
+                             G, I, H, w_stride, stream);
+}
+
+extern "C" int om_merged_mlp_row_dot_parts(int I) {
+    if (I < ROW_DOT_COLS || I % ROW_DOT_COLS != 0) return OM_ERR_SHAPE;
+    return I / ROW_DOT_COLS;
+}
+
+extern "C" int om_merged_mlp_down_dgrad_weighted(const void *dy, const int32_t *dy_rows, int64_t src_rows,
+                                                 const void *w_down, const void *g, const void *u,
+                                                 const float *row_weights, void *dg, void *du,
+                                                 float *row_dot, const int32_t *cum_token_counts,
+                                                 int64_t rows, int G, int I, int H, int64_t w_stride,
+                                                 void *stream) {
+    if (rows > 0 && (!dy_rows || !row_weights || !row_dot)) return OM_ERR_NULL;
+    if (src_rows < 1 && rows > 0) return OM_ERR_SHAPE;
+    return down_dgrad_launch(dy, dy_rows, src_rows, w_down, g, u, row_weights, dg, du, row_dot,
+                             cum_token_counts, rows, G, I, H, w_stride, stream);
 }
 
 extern "C" int om_merged_mlp_gate_up_dgrad(const void *dg, const void *du, const void *w_gate,

@@ -168,6 +168,42 @@ __global__ __launch_bounds__(256) void combine_backward_kernel(
     if (lane == 0) Elem<TW>::store(dw + static_cast<int64_t>(t) * K + k, acc);
 }
 
+// The routing weight of every sorted row, for expert kernels that apply it themselves: routed
+// entry rt -> row pos = output_indices[rt], token t = input_indices[pos], slot k = sel_idx[rt];
+// row_weights[pos] = w[t,k].
+template <typename TW>
+__global__ __launch_bounds__(256) void row_weights_kernel(
+    const TW *__restrict__ routing_weights, const int32_t *__restrict__ selected_experts_indices,
+    const int32_t *__restrict__ input_indices, const int32_t *__restrict__ output_indices,
+    float *__restrict__ row_weights, int64_t RT, int K) {
+    const int64_t rt = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (rt >= RT) return;
+    const int32_t pos = output_indices[rt];
+    const int32_t t = input_indices[pos];
+    row_weights[pos] = Elem<TW>::load(routing_weights + static_cast<int64_t>(t) * K + selected_experts_indices[rt]);
+}
+
+// The way back: dw[t,k] = sum over the `parts` column ranges of row_dot[part][pos], added in order.
+template <typename TW>
+__global__ __launch_bounds__(256) void row_weights_grad_kernel(
+    const float *__restrict__ row_dot, int parts, const int32_t *__restrict__ selected_experts_indices,
+    const int32_t *__restrict__ input_indices, const int32_t *__restrict__ output_indices,
+    TW *__restrict__ dw, int64_t RT, int K) {
+    const int64_t rt = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (rt >= RT) return;
+    const int32_t pos = output_indices[rt];
+    const int32_t t = input_indices[pos];
+    float s = 0.0f;
+    for (int p0 = 0; p0 < parts; p0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = (p0 + u < parts) ? row_dot[(p0 + u) * RT + pos] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; u++) s += v[u];
+    }
+    Elem<TW>::store(dw + static_cast<int64_t>(t) * K + selected_experts_indices[rt], s);
+}
+
 // output[indices[c],:] += input[c,:], atomically per element so duplicate indices add up.
 __global__ void index_add_f32_kernel(const float *__restrict__ input, float *__restrict__ output,
                                      const int32_t *__restrict__ indices, int64_t C, int64_t E) {
@@ -323,6 +359,58 @@ extern "C" int om_reduce_ggemm_output_residual(const void *ggemm_output, const v
     return reduce_ggemm_output_launch(ggemm_output, routing_weights, cum_expert_counts_ep,
                                       selected_experts_indices, output_indices, final_hidden_states, T, K,
                                       E, dtype, weights_dtype, 0, residual, stream);
+}
+
+extern "C" int om_sum_ggemm_output(const void *ggemm_output, const int32_t *cum_expert_counts_ep,
+                                   const int32_t *output_indices, const void *residual,
+                                   void *final_hidden_states, int64_t T, int64_t E, int dtype,
+                                   void *stream) {
+    return reduce_ggemm_output_launch(ggemm_output, nullptr, cum_expert_counts_ep, nullptr, output_indices,
+                                      final_hidden_states, T, 0, E, dtype, OM_F32, 1, residual, stream);
+}
+
+extern "C" int om_moe_row_weights(const void *routing_weights, const int32_t *selected_experts_indices,
+                                  const int32_t *input_indices, const int32_t *output_indices,
+                                  float *row_weights, int64_t RT, int K, int weights_dtype, void *stream) {
+    if (weights_dtype != OM_F32 && weights_dtype != OM_BF16) return OM_ERR_DTYPE;
+    if (RT < 0 || K < 1 || RT > 0x7fffffffLL) return OM_ERR_SHAPE;
+    if (RT == 0) return OM_OK;
+    if (!routing_weights || !selected_experts_indices || !input_indices || !output_indices || !row_weights)
+        return OM_ERR_NULL;
+    hipStream_t st = om_stream(stream);
+    const unsigned nb = static_cast<unsigned>((RT + 255) / 256);
+    if (weights_dtype == OM_F32)
+        row_weights_kernel<float><<<nb, 256, 0, st>>>(static_cast<const float *>(routing_weights),
+                                                      selected_experts_indices, input_indices,
+                                                      output_indices, row_weights, RT, K);
+    else
+        row_weights_kernel<uint16_t><<<nb, 256, 0, st>>>(static_cast<const uint16_t *>(routing_weights),
+                                                         selected_experts_indices, input_indices,
+                                                         output_indices, row_weights, RT, K);
+    return om_launch_status();
+}
+
+extern "C" int om_moe_row_weights_grad(const float *row_dot, int parts,
+                                       const int32_t *selected_experts_indices,
+                                       const int32_t *input_indices, const int32_t *output_indices,
+                                       void *routing_weights_grad, int64_t RT, int K, int weights_dtype,
+                                       void *stream) {
+    if (weights_dtype != OM_F32 && weights_dtype != OM_BF16) return OM_ERR_DTYPE;
+    if (RT < 0 || K < 1 || parts < 1 || RT > 0x7fffffffLL) return OM_ERR_SHAPE;
+    if (RT == 0) return OM_OK;
+    if (!row_dot || !selected_experts_indices || !input_indices || !output_indices || !routing_weights_grad)
+        return OM_ERR_NULL;
+    hipStream_t st = om_stream(stream);
+    const unsigned nb = static_cast<unsigned>((RT + 255) / 256);
+    if (weights_dtype == OM_F32)
+        row_weights_grad_kernel<float><<<nb, 256, 0, st>>>(row_dot, parts, selected_experts_indices,
+                                                           input_indices, output_indices,
+                                                           static_cast<float *>(routing_weights_grad), RT, K);
+    else
+        row_weights_grad_kernel<uint16_t><<<nb, 256, 0, st>>>(row_dot, parts, selected_experts_indices,
+                                                              input_indices, output_indices,
+                                                              static_cast<uint16_t *>(routing_weights_grad), RT, K);
+    return om_launch_status();
 }
 
 extern "C" int om_reduce_ggemm_output_backward(

@@ -97,6 +97,21 @@ SIGNATURES = {
                                                    c_int, c_i64, c_void_p]),
     "om_grouped_gemm_wgrad_gathered": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p,
                                                c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
+    "om_moe_row_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
+                                   c_void_p]),
+    "om_merged_mlp_gate_up_fwd_weighted": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p,
+                                                   c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int,
+                                                   c_int, c_int, c_i64, c_void_p]),
+    "om_sum_ggemm_output": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int,
+                                    c_void_p]),
+    "om_grouped_gemm_wgrad_gathered_out": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p,
+                                                   c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
+    "om_merged_mlp_row_dot_parts": (c_int, [c_int]),
+    "om_merged_mlp_down_dgrad_weighted": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p,
+                                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64,
+                                                  c_int, c_int, c_int, c_i64, c_void_p]),
+    "om_moe_row_weights_grad": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_i64,
+                                        c_int, c_int, c_void_p]),
     "om_merged_mlp_down_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
     "om_merged_mlp_gate_up_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -115,7 +130,8 @@ launch_log = None
 launch_filter = None   # optional set of entry-point names: only these are timed while launch_log is set
 _UNTIMED = {"om_version", "om_arch", "om_strerror", "om_moe_sort_workspace_bytes",
             "om_router_balance_workspace_bytes", "om_rmsnorm_bwd_workspace_bytes",
-            "om_router_gate_wgrad_workspace_bytes", "om_router_gate_logits_split_workspace_bytes"}
+            "om_router_gate_wgrad_workspace_bytes", "om_router_gate_logits_split_workspace_bytes",
+            "om_merged_mlp_row_dot_parts"}
 
 
 class NativeLibraryError(RuntimeError):

@@ -579,6 +579,171 @@ class GatheredGroupMLPFunction(torch.autograd.Function):
         return (hidden_states_grad, None, None, None, None, *flat)
 
 
+def routed_mlp_kernel_fits(hidden_states, routing_weights, w_gate, w_down):
+    """True when RoutedMLPFunction's kernels take these operands: bf16 activations and expert
+    weights on the GPU, fp32 or bf16 routing weights, H and I multiples of 128."""
+    G, I, H = w_gate.shape
+    return (hidden_states.is_cuda and hidden_states.dim() == 2
+            and hidden_states.dtype == torch.bfloat16 and w_gate.dtype == torch.bfloat16
+            and w_down.dtype == torch.bfloat16
+            and routing_weights.dtype in (torch.bfloat16, torch.float32)
+            and H % 128 == 0 and I % 128 == 0)
+
+
+def _routed_mlp_forward(hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                        output_indices, selected_experts_indices, w_gate, w_up, w_down,
+                        cum_token_counts, residual):
+    """-> (final [T,H], cum, g, u, h, row_weights): gather, weighted SwiGLU MLP, unweighted sum."""
+    _n.require_cuda_contiguous(hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                               output_indices, selected_experts_indices, residual)
+    _require_bf16(hidden_states, w_gate, w_up, w_down)
+    T, H = hidden_states.shape
+    K = routing_weights.shape[1]
+    rows = input_indices.shape[0]
+    G, I, _ = w_gate.shape
+    dev, dt = hidden_states.device, hidden_states.dtype
+    cum = _device_counts(cum_token_counts, dev)
+    lib, st = _n.lib(), _n.stream()
+    sgu = _expert_stride(w_gate)
+    if _expert_stride(w_up) != sgu:
+        raise _n.NativeLibraryError("gate and up expert weights must share one expert pitch")
+    row_weights = torch.empty((rows,), dtype=torch.float32, device=dev)
+    g = torch.empty((rows, I), dtype=dt, device=dev)
+    u = torch.empty_like(g)
+    h = torch.empty_like(g)
+    y = torch.empty((rows, H), dtype=dt, device=dev)
+    final = torch.empty((T, H), dtype=dt, device=dev)
+    with record_pcl_function("1moeblock--7gmlp_fwd"):
+        _n.check(lib.om_moe_row_weights(
+            _n.ptr(routing_weights), _n.ptr(selected_experts_indices), _n.ptr(input_indices),
+            _n.ptr(output_indices), _n.ptr(row_weights), rows, K, _n.dtype_code(routing_weights), st),
+            "om_moe_row_weights")
+        _n.check(lib.om_merged_mlp_gate_up_fwd_weighted(
+            _n.ptr(hidden_states), _n.ptr(input_indices), T, _n.ptr(w_gate), _n.ptr(w_up),
+            _n.ptr(row_weights), _n.ptr(g), _n.ptr(u), _n.ptr(h), _n.ptr(cum), rows, G, I, H, sgu, st),
+            "om_merged_mlp_gate_up_fwd_weighted")
+        _n.check(lib.om_grouped_gemm_fwd(
+            _n.ptr(h), _n.ptr(w_down), _n.ptr(y), _n.ptr(cum), rows, G, H, I, _expert_stride(w_down), st),
+            "om_grouped_gemm_fwd")
+    with record_pcl_function("1moeblock--8gmlp_output_reduction_fwd"):
+        _n.check(lib.om_sum_ggemm_output(
+            _n.ptr(y), _n.ptr(cum_expert_counts_ep), _n.ptr(output_indices), _n.ptr(residual),
+            _n.ptr(final), T, H, _n.dtype_code(final), st), "om_sum_ggemm_output")
+    return final, cum, g, u, h, row_weights
+
+
+def _routed_mlp_backward(dfinal, hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                         output_indices, selected_experts_indices, w_gate, w_up, w_down, cum, g, u, h,
+                         row_weights):
+    """-> (hidden_states_grad, routing_weights_grad, dw_gate, dw_up, dw_down)."""
+    dfinal = dfinal.contiguous()
+    T, H = hidden_states.shape
+    K = routing_weights.shape[1]
+    rows = input_indices.shape[0]
+    G, I, _ = w_gate.shape
+    dev, dt = hidden_states.device, hidden_states.dtype
+    lib, st = _n.lib(), _n.stream()
+    dg = torch.empty_like(g)
+    du = torch.empty_like(u)
+    dx_rows = torch.empty((rows, H), dtype=dt, device=dev)
+    dw_gate = torch.empty((G, I, H), dtype=dt, device=dev)
+    dw_up = torch.empty((G, I, H), dtype=dt, device=dev)
+    dw_down = torch.empty((G, H, I), dtype=dt, device=dev)
+    # the kernel writes the entry of every routed (token, k) pair; pairs outside the expert window
+    # stay zero
+    if rows == routing_weights.numel():
+        routing_weights_grad = torch.empty_like(routing_weights)
+    else:
+        routing_weights_grad = torch.zeros_like(routing_weights)
+    hidden_states_grad = torch.empty_like(hidden_states)
+    with record_pcl_function("1moeblock--7gmlp_bwd"):
+        if rows > 0:
+            parts = lib.om_merged_mlp_row_dot_parts(I)
+            if parts < 1:
+                _n.check(parts, "om_merged_mlp_row_dot_parts")
+            row_dot = torch.empty((parts, rows), dtype=torch.float32, device=dev)
+            _n.check(lib.om_grouped_gemm_wgrad_gathered_out(
+                _n.ptr(dfinal), _n.ptr(input_indices), T, _n.ptr(h), _n.ptr(dw_down), _n.ptr(cum), rows,
+                G, H, I, 0, st), "om_grouped_gemm_wgrad_gathered_out(down)")
+            _n.check(lib.om_merged_mlp_down_dgrad_weighted(
+                _n.ptr(dfinal), _n.ptr(input_indices), T, _n.ptr(w_down), _n.ptr(g), _n.ptr(u),
+                _n.ptr(row_weights), _n.ptr(dg), _n.ptr(du), _n.ptr(row_dot), _n.ptr(cum), rows, G, I, H,
+                _expert_stride(w_down), st), "om_merged_mlp_down_dgrad_weighted")
+            _n.check(lib.om_moe_row_weights_grad(
+                _n.ptr(row_dot), parts, _n.ptr(selected_experts_indices), _n.ptr(input_indices),
+                _n.ptr(output_indices), _n.ptr(routing_weights_grad), rows, K,
+                _n.dtype_code(routing_weights_grad), st), "om_moe_row_weights_grad")
+            for grad, dw, name in ((dg, dw_gate, "gate"), (du, dw_up, "up")):
+                _n.check(lib.om_grouped_gemm_wgrad_gathered(
+                    _n.ptr(grad), _n.ptr(hidden_states), _n.ptr(input_indices), T, _n.ptr(dw), _n.ptr(cum),
+                    rows, G, I, H, 0, st), f"om_grouped_gemm_wgrad_gathered({name})")
+            _n.check(lib.om_merged_mlp_gate_up_dgrad(
+                _n.ptr(dg), _n.ptr(du), _n.ptr(w_gate), _n.ptr(w_up), _n.ptr(dx_rows), _n.ptr(cum), rows,
+                G, I, H, _expert_stride(w_gate), st), "om_merged_mlp_gate_up_dgrad")
+        else:   # nothing routed to these experts: the weight gradients are zero
+            for dw, n_, k_ in ((dw_down, H, I), (dw_gate, I, H), (dw_up, I, H)):
+                _n.check(lib.om_grouped_gemm_wgrad(None, None, _n.ptr(dw), _n.ptr(cum), 0, G, n_, k_, 0, st),
+                         "om_grouped_gemm_wgrad(empty)")
+    with record_pcl_function("1moeblock--6gmlp_input_prep_bwd"):
+        pcl_xpu_customops.shuffle_sub_matrix_reduce(dx_rows, cum_expert_counts_ep, output_indices,
+                                                    hidden_states_grad)
+    return hidden_states_grad, routing_weights_grad, dw_gate, dw_up, dw_down
+
+
+class RoutedMLPFunction(torch.autograd.Function):
+    """The expert half of the block in one function: PrepareInputForGroupGemmFunction, the SwiGLU
+    MLP of every expert and GroupGemmOutputReductionFunction (reference moe.py:217-405), with both
+    row permutations and the routing weight folded into the GEMMs:
+
+      forward   h = w[t,k] * silu(x Wg^T) * (x Wu^T) formed in the gate+up epilogue (x read through
+                input_indices), y = h Wd^T, final[t] = (residual[t] +) sum of the token's rows of y;
+      backward  the down projection's two backward GEMMs read dfinal through input_indices, the
+                SwiGLU-backward epilogue applies w and forms the routing weights' gradient
+                sum_i (dfinal Wd)[i] * silu(g)[i] * u[i]; the rest as GatheredMergedMLPFunction.
+
+    Neither the gathered input, nor the experts' output gradient w[t,k] * dfinal[t] (both [rows, H])
+    is written.  The weight commutes with the linear down projection, so this is the reference's
+    mathematics; h is rounded to bf16 after the weight instead of before, so results agree with the
+    separate functions to bf16 accuracy, not bit for bit.
+
+    `weights`: (gate, up, down) as [G, I, H] / [G, H, I] tensors when n_merged is true, else the
+    3*G per-expert matrices of GroupMLPFunction."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, routing_weights, input_indices, cum_expert_counts_ep, output_indices,
+                selected_experts_indices, cum_token_counts, residual, n_merged, *weights):
+        if n_merged:
+            wg, wu, wd = weights
+        else:
+            N = len(weights) // 3
+            wg, wu, wd = [_strided_expert_view([weights[3 * n + j] for n in range(N)]) for j in range(3)]
+        hidden_states = hidden_states.contiguous()
+        routing_weights = routing_weights.contiguous()
+        if residual is not None:
+            residual = residual.contiguous()
+        final, cum, g, u, h, row_weights = _routed_mlp_forward(
+            hidden_states, routing_weights, input_indices, cum_expert_counts_ep, output_indices,
+            selected_experts_indices, wg, wu, wd, cum_token_counts, residual)
+        ctx.save_for_backward(hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                              output_indices, selected_experts_indices, wg, wu, wd, cum, g, u, h,
+                              row_weights)
+        ctx.n_merged = bool(n_merged)
+        ctx.has_residual = residual is not None
+        return final
+
+    @staticmethod
+    def backward(ctx, dfinal):
+        dx, drw, dwg, dwu, dwd = _routed_mlp_backward(dfinal, *ctx.saved_tensors)
+        if ctx.n_merged:
+            wgrads = (dwg, dwu, dwd)
+        else:
+            wgrads = []
+            for n in range(dwg.shape[0]):
+                wgrads += [dwg[n], dwu[n], dwd[n]]
+        return (dx, drw, None, None, None, None, None, dfinal if ctx.has_residual else None, None,
+                *wgrads)
+
+
 def _strided_expert_view(weights):
     """[G, out, in] view over per-expert matrices that lie at a constant pitch in one storage."""
     w0 = weights[0]
@@ -758,12 +923,15 @@ class MergedMLP(nn.Module):
 
 def expert_computation(hidden_states, routing_weights, selected_experts, expert_start_idx,
                        expert_end_idx, experts_fn, num_total_experts, gathered_experts_fn=None,
-                       residual=None):
+                       residual=None, routed_experts_fn=None):
     """K1..K6 for 2-D hidden_states [T,H]: permute, run `experts_fn(ggemm_input, cum_token_counts)`,
     combine.  Shared by the OLMoE and DeepSeek-V3 blocks.  With `gathered_experts_fn(hidden_states,
     input_indices, cum_expert_counts_ep, output_indices, cum_token_counts)` the experts read the
     tokens through the index and K4's gathered copy is not built.  With `residual` [T,H] the result
-    is residual + combine(...), added inside the combine kernel."""
+    is residual + combine(...), added inside the combine kernel.  `routed_experts_fn(hidden_states,
+    routing_weights, input_indices, cum_expert_counts_ep, output_indices, selected_experts_indices,
+    cum_token_counts, residual)` may do gather, experts and combine in one function
+    (RoutedMLPFunction); it returns None when its kernels do not take the operands."""
     T, K = selected_experts.shape
     with record_pcl_function("1moeblock--3index_calculation"):
         (cum_token_counts, cum_expert_counts_ep, input_indices, output_indices,
@@ -776,6 +944,11 @@ def expert_computation(hidden_states, routing_weights, selected_experts, expert_
     input_indices = input_indices[:num_routed_tokens]
     output_indices = output_indices[:num_routed_tokens]
     selected_experts_indices = selected_experts_indices[:num_routed_tokens]
+    if routed_experts_fn is not None:
+        final = routed_experts_fn(hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                                  output_indices, selected_experts_indices, cum_token_counts, residual)
+        if final is not None:
+            return final
     if gathered_experts_fn is not None:
         ggemm_output = gathered_experts_fn(hidden_states, input_indices, cum_expert_counts_ep,
                                            output_indices, cum_token_counts)
@@ -829,6 +1002,9 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
         self.router_logits_fp32 = bool(getattr(config, "router_logits_fp32", False))
         # merged experts read the tokens through input_indices instead of a gathered copy
         self.fuse_input_gather = bool(getattr(config, "fuse_input_gather", True))
+        # the routing weight is applied inside the expert MLP and the combine's backward is folded
+        # into the down projection's backward GEMMs (RoutedMLPFunction); needs fuse_input_gather
+        self.fuse_routing_weights = bool(getattr(config, "fuse_routing_weights", True))
 
     def _experts_fn(self, ggemm_input, cum_token_counts):
         if isinstance(self.experts, MergedMLP):
@@ -850,6 +1026,27 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
             mlp_params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
         return GatheredGroupMLPFunction.apply(hidden_states, input_indices, cum_expert_counts_ep,
                                               output_indices, cum_token_counts, *mlp_params)
+
+    def _routed_experts_fn(self, hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                           output_indices, selected_experts_indices, cum_token_counts, residual):
+        if isinstance(self.experts, MergedMLP):
+            weights = (self.experts.gate_proj_merged_weight, self.experts.up_proj_merged_weight,
+                       self.experts.down_proj_merged_weight)
+            if not routed_mlp_kernel_fits(hidden_states, routing_weights, weights[0], weights[2]):
+                return None
+            return RoutedMLPFunction.apply(hidden_states, routing_weights, input_indices,
+                                           cum_expert_counts_ep, output_indices, selected_experts_indices,
+                                           cum_token_counts, residual, True, *weights)
+        pack_expert_weights(self.experts)
+        w0, d0 = self.experts[0].gate_proj.weight, self.experts[0].down_proj.weight
+        if not routed_mlp_kernel_fits(hidden_states, routing_weights, w0.unsqueeze(0), d0.unsqueeze(0)):
+            return None
+        mlp_params = []
+        for expert in self.experts:
+            mlp_params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
+        return RoutedMLPFunction.apply(hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                                       output_indices, selected_experts_indices, cum_token_counts,
+                                       residual, False, *mlp_params)
 
     def forward_with_residual(self, hidden_states, residual):
         """(residual + forward(hidden_states)[0], router_logits): the decoder layer's
@@ -876,10 +1073,12 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
         def expert_computation_block(hidden_states, selected_experts, routing_weights, residual=None):
             b, s, h = hidden_states.shape
             gathered = self._gathered_experts_fn if self.fuse_input_gather else None
+            routed = self._routed_experts_fn if (self.fuse_input_gather and self.fuse_routing_weights) else None
             out = expert_computation(hidden_states.reshape(-1, h), routing_weights, selected_experts,
                                      self.expert_start_idx, self.expert_end_idx, self._experts_fn,
                                      self.num_experts, gathered_experts_fn=gathered,
-                                     residual=None if residual is None else residual.reshape(-1, h))
+                                     residual=None if residual is None else residual.reshape(-1, h),
+                                     routed_experts_fn=routed)
             return out.reshape(b, s, h)
 
         args = [hidden_states, selected_experts, routing_weights]

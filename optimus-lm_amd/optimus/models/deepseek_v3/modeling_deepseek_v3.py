@@ -149,16 +149,33 @@ class DeepseekV3ParallelMoE(nn.Module):
         return _moe.GatheredGroupMLPFunction.apply(hidden_states, input_indices, cum_expert_counts_ep,
                                                    output_indices, cum_token_counts, *params)
 
+    def _routed_experts_fn(self, hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                           output_indices, selected_experts_indices, cum_token_counts, residual):
+        _moe.pack_expert_weights(self.experts)
+        w0, d0 = self.experts[0].gate_proj.weight, self.experts[0].down_proj.weight
+        if not _moe.routed_mlp_kernel_fits(hidden_states, routing_weights, w0.unsqueeze(0), d0.unsqueeze(0)):
+            return None
+        params = []
+        for expert in self.experts:
+            params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
+        return _moe.RoutedMLPFunction.apply(hidden_states, routing_weights, input_indices,
+                                            cum_expert_counts_ep, output_indices, selected_experts_indices,
+                                            cum_token_counts, residual, False, *params)
+
     def moe(self, hidden_states, topk_indices, topk_weights, residual=None):
         """Routed part for [T,H] hidden_states (reference :221-244): fp32 weights, fp32 sum over a
         token's local experts, one rounding to the activation dtype.  The local experts read their
-        tokens through the permutation index (no gathered copy of the activations).  `residual`
-        [T,H] is added to the rounded result inside the combine kernel."""
-        gathered = self._gathered_experts_fn if getattr(self.config, "fuse_input_gather", True) else None
+        tokens through the permutation index (no gathered copy of the activations) and apply the
+        routing weight themselves (RoutedMLPFunction) unless the config switches that off.
+        `residual` [T,H] is added to the rounded result inside the combine kernel."""
+        fuse_gather = getattr(self.config, "fuse_input_gather", True)
+        gathered = self._gathered_experts_fn if fuse_gather else None
+        routed = self._routed_experts_fn if (
+            fuse_gather and getattr(self.config, "fuse_routing_weights", True)) else None
         return _moe.expert_computation(hidden_states, topk_weights, topk_indices,
                                        self.expert_start_idx, self.expert_end_idx, self._experts_fn,
                                        self.config.n_routed_experts, gathered_experts_fn=gathered,
-                                       residual=residual)
+                                       residual=residual, routed_experts_fn=routed)
 
     def forward(self, hidden_states):
         topk_indices, topk_weights = self.gate(hidden_states)

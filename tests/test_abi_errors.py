@@ -154,6 +154,39 @@ def test_grouped_gemms(lib):
     assert lib.om_grouped_gemm_wgrad_gathered(P, P, P, 16384, ODD, P, *g) == ALIGN
 
 
+def test_routing_weight_folded_into_the_expert_mlp(lib):
+    g = (131072, 64, 1024, 2048, 0, None)
+    assert lib.om_moe_row_weights(P, P, P, P, P, 131072, 8, 7, None) == DTYPE
+    assert lib.om_moe_row_weights(P, P, P, P, None, 131072, 8, F32, None) == NULL
+    assert lib.om_moe_row_weights(P, P, P, P, P, 131072, 0, F32, None) == SHAPE
+    assert lib.om_moe_row_weights(None, None, None, None, None, 0, 8, BF16, None) == OK
+    assert lib.om_merged_mlp_gate_up_fwd_weighted(P, P, 16384, P, P, None, P, P, P, P, *g) == NULL   # no weights
+    assert lib.om_merged_mlp_gate_up_fwd_weighted(P, None, 16384, P, P, P, P, P, P, P, *g) == NULL   # no index
+    assert lib.om_merged_mlp_gate_up_fwd_weighted(P, P, 0, P, P, P, P, P, P, P, *g) == SHAPE
+    assert lib.om_merged_mlp_gate_up_fwd_weighted(P, P, 16384, P, P, P, P, P, P, P, 131072, 64, 1000, 2048, 0, None) == SHAPE
+    assert lib.om_merged_mlp_gate_up_fwd_weighted(P, None, 0, P, P, None, P, P, P, P, 0, 64, 1024, 2048, 0, None) == OK
+    assert lib.om_sum_ggemm_output(P, None, P, None, P, 16384, 2048, BF16, None) == NULL
+    assert lib.om_sum_ggemm_output(P, P, P, None, P, 16384, 2048, 7, None) == DTYPE
+    assert lib.om_sum_ggemm_output(P, P, P, None, P, 0, 2048, BF16, None) == OK
+    gw = (131072, 64, 2048, 1024, 0, None)
+    assert lib.om_grouped_gemm_wgrad_gathered_out(P, None, 16384, P, P, P, *gw) == NULL
+    assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 0, P, P, P, *gw) == SHAPE
+    assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 1 << 21, P, P, P, *gw) == SHAPE   # source > 2^31 elements
+    assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 16384, P, ODD, P, *gw) == ALIGN
+    assert lib.om_merged_mlp_row_dot_parts(1024) == 16
+    assert lib.om_merged_mlp_row_dot_parts(100) == SHAPE
+    assert lib.om_merged_mlp_down_dgrad_weighted(P, P, 16384, P, P, P, P, P, P, None, P, *g) == NULL   # no row_dot
+    assert lib.om_merged_mlp_down_dgrad_weighted(P, P, 16384, P, P, P, None, P, P, P, P, *g) == NULL   # no weights
+    assert lib.om_merged_mlp_down_dgrad_weighted(P, None, 16384, P, P, P, P, P, P, P, P, *g) == NULL   # no index
+    assert lib.om_merged_mlp_down_dgrad_weighted(P, P, 0, P, P, P, P, P, P, P, P, *g) == SHAPE
+    assert lib.om_merged_mlp_down_dgrad_weighted(P, P, 16384, P, P, P, P, ODD, P, P, P, *g) == ALIGN
+    assert lib.om_merged_mlp_down_dgrad_weighted(P, None, 0, P, P, P, None, P, P, None, P, 0, 64, 1024, 2048, 0, None) == OK
+    assert lib.om_moe_row_weights_grad(P, 0, P, P, P, P, 131072, 8, F32, None) == SHAPE
+    assert lib.om_moe_row_weights_grad(None, 16, P, P, P, P, 131072, 8, F32, None) == NULL
+    assert lib.om_moe_row_weights_grad(P, 16, P, P, P, P, 131072, 8, 9, None) == DTYPE
+    assert lib.om_moe_row_weights_grad(None, 16, None, None, None, None, 0, 8, F32, None) == OK
+
+
 def test_check_raises_with_the_library_text():
     with pytest.raises(n.NativeLibraryError, match="dtype"):
         n.check(DTYPE, "om_adamw_step")

@@ -217,6 +217,18 @@ def test_unmerged_block_matches_merged(cuda):
     b = _olmoe_block(inp, cuda, fast=False, fp32_logits=False)
     d = _olmoe_block(inp, cuda, fast=True, merged=False, fp32_logits=False)
     x = inp["x"].to(cuda).view(2, c["T"] // 2, c["H"])
+    # merged and per-expert weights give the same bits with the routing weight folded into the MLP
+    fused = []
+    for blk in (a, d):
+        xi = x.clone().requires_grad_(True)
+        o, _ = blk(xi)
+        o.backward(inp["dout"].to(cuda).view_as(o))
+        fused.append((o, xi.grad))
+        blk.zero_grad()
+    assert torch.equal(fused[0][0], fused[1][0]) and torch.equal(fused[0][1], fused[1][1])
+    # the slow block keeps the reference's sequence gather -> experts -> weighted combine; the fast
+    # blocks give its bits when their fusion of the routing weight is switched off
+    a.fuse_routing_weights = d.fuse_routing_weights = False
     outs = []
     for blk in (a, b, d):
         xi = x.clone().requires_grad_(True)
@@ -266,6 +278,7 @@ def test_gather_fusion_switch_changes_no_bit(cuda, name, merged):
         blk = _olmoe_block(inp, cuda, merged=merged)
         assert blk.fuse_input_gather is True
         blk.fuse_input_gather = fuse
+        blk.fuse_routing_weights = False   # that fusion moves roundings; it has its own tests
         xi = inp["x"].to(cuda).view(1, c["T"], c["H"]).requires_grad_(True)
         o, _ = blk(xi)
         o.backward(inp["dout"].to(cuda).view_as(o))
