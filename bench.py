@@ -36,10 +36,12 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # counters cannot be collected inside the timed run.
 MIB = float(1 << 20)
 MEASURED_TRAFFIC_BYTES = {
-    "om_merged_mlp_gate_up_fwd": (3220 + 768) * MIB, "om_grouped_gemm_fwd": (1403 + 512) * MIB,
+    "om_merged_mlp_gate_up_fwd": (3220 + 768) * MIB, "om_grouped_gemm_fwd": (1389 + 512) * MIB,
     "om_grouped_gemm_wgrad": (927 + 256) * MIB, "om_merged_mlp_down_dgrad": (1952 + 512) * MIB,
-    "om_merged_mlp_gate_up_dgrad": (3449 + 512) * MIB, "om_adamw_step": (92125 + 92125) * MIB,
-    "om_merged_mlp_gate_up_fwd_gathered": (3288 + 768) * MIB, "om_grouped_gemm_wgrad_gathered": (962 + 256) * MIB,
+    "om_merged_mlp_gate_up_dgrad": (3480 + 512) * MIB, "om_adamw_step": (92125 + 92125) * MIB,
+    "om_merged_mlp_gate_up_fwd_gathered": (3288 + 768) * MIB, "om_grouped_gemm_wgrad_gathered": (989 + 256) * MIB,
+    "om_merged_mlp_gate_up_fwd_weighted": (3241 + 768) * MIB, "om_grouped_gemm_wgrad_gathered_out": (903 + 256) * MIB,
+    "om_merged_mlp_down_dgrad_weighted": (1927 + 523) * MIB,
 }
 
 GEMM_ENTRY_PRODUCTS = {     # C-ABI entry -> number of [rows x N x K] products per launch
