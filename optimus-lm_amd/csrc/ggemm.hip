@@ -231,6 +231,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // stage does not depend on the loads in flight to the other
     __shared__ __attribute__((aligned(1024))) char stage0[A_BYTES + B_BYTES];
     __shared__ __attribute__((aligned(1024))) char stage1[A_BYTES + B_BYTES];
+    // wgrad through an index: the current expert's slice of the index is kept in LDS (filled when
+    // the block moves to another expert) for the look-up that a tile's first loads wait for; the
+    // look-ups inside the main loop run one step ahead and go to global memory (reading them from
+    // LDS measured 20 % slower: they queue with the fragment reads)
+    constexpr bool GATHER_W = GATHER == GATHER_B || GATHER == GATHER_WA;
+    constexpr int IDX_CACHE = GATHER_W ? (BM == 256 ? 4096 : 2048) : 1;
+    __shared__ int idx_cache[IDX_CACHE];
+    int cached_expert = -1;
     __shared__ int tile_end[EPI == EPI_WGRAD ? 1 : MAX_EXPERTS];   // see build_tile_table
     __shared__ int seg[EPI == EPI_WGRAD ? 1 : MAX_EXPERTS + 1];
 
@@ -279,16 +287,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     const int lda32 = static_cast<int>(p.lda), ldb32 = static_cast<int>(p.ldb);
     // GATHER_B: the B rows that contraction step `step` needs, looked up one step ahead of the
     // loads that use them (plain loads: they land before the next wait for the direct loads).
+    auto index_of = [&](int step, int c0, int c) -> int {   // c0: the step's first row (block-uniform)
+        if (step == 0 && c0 + BK <= IDX_CACHE) return idx_cache[GATHER_W ? c : 0];
+        return p.row_index[c_begin + c];
+    };
     auto load_b_src = [&](int step) {
         if (GATHER != GATHER_B || step >= loop_steps) return;
         const int c0 = (step < steps_per_phase ? rotated(step) : step) * BK;
-        // One 4-byte load per B load (measured faster than one load per wavefront plus lane
-        // permutes, which queue behind the fragment reads).  Kept as loaded: any arithmetic on the
-        // value here would put the wait for the load here too.
+        // One 4-byte read per B load (measured faster than one read per wavefront plus lane
+        // permutes, which queue behind the fragment reads).  Kept as read: any arithmetic on the
+        // value here would put the wait for it here too.
 #pragma unroll
         for (int i = 0; i < B_LOADS; i++) {
             const int c = min(c0 + b_crow[i], c_len - 1);   // past the segment: any valid row (A is zeroed)
-            b_src[GATHER == GATHER_B ? i : 0] = p.row_index[c_begin + c];
+            b_src[GATHER == GATHER_B ? i : 0] = index_of(step, c0, c);
         }
     };
 
@@ -298,7 +310,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 #pragma unroll
         for (int i = 0; i < A_LOADS; i++) {
             const int c = min(c0 + a_crow[i], c_len - 1);   // past the segment: any valid row (zeroed in LDS)
-            a_src[GATHER == GATHER_WA ? i : 0] = p.row_index[c_begin + c];
+            a_src[GATHER == GATHER_WA ? i : 0] = index_of(step, c0, c);
         }
     };
 
@@ -383,6 +395,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                 const int ch = (lane_s % CPR) ^ ((b_crow[i] & 3) << 2);
                 b_off[i] = static_cast<int>((EPI == EPI_WGRAD ? 0 : expert * p.strideB) + n0 + ch * 8);
             }
+        }
+        if (GATHER_W && expert != cached_expert) {
+            // every wavefront is past the barrier that ends the previous tile's main loop, so no
+            // one still reads the cache; `expert` is block-uniform, so all take this branch together
+            const int n_cached = min(c_len, IDX_CACHE);
+            for (int i = tid; i < n_cached; i += NW * 64) idx_cache[GATHER_W ? i : 0] = p.row_index[c_begin + i];
+            cached_expert = expert;
+            __syncthreads();
         }
         load_b_src(0);
         load_a_src(0);
