@@ -196,3 +196,37 @@ def test_block_switch_for_routing_weight_fusion(cuda, merged):
         assert mean_rel(a.float().cpu(), b.float().cpu()) <= 1e-2
         differs = differs or not torch.equal(a, b)
     assert differs   # the switch really selects another code path
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_routed_mlp_random_shapes(cuda, seed):
+    """Seeded sweep over token counts, top-k, expert windows and sizes.  With unit routing weights
+    the folded form must give the separate functions' bits (this pins the two gathered backward
+    GEMMs and the row bookkeeping); with random weights it must stay within bf16 accuracy of them
+    and give exact zeros for pairs outside the expert window."""
+    import numpy as np
+    rng = np.random.RandomState(4321 + seed)
+    N = int(rng.choice([4, 8, 16, 64]))
+    K = int(rng.choice([1, 2, min(4, N)]))
+    T = int(rng.choice([5, 64, 300, 1024, 5000]))
+    H = int(rng.choice([128, 256, 384, 512]))
+    I = int(rng.choice([128, 256, 384]))
+    start = int(rng.choice([0, N // 4]))
+    end = int(rng.choice([N, max(start + 1, N - N // 4)]))
+    wdt = [torch.float32, torch.bfloat16][seed % 2]
+    c = _case(T, K, N, start, end, I, H, float(rng.choice([0.0, 1.0])), cuda, weights_dtype=wdt, seed=seed)
+    tag = (T, K, N, start, end, I, H, c["rows"])
+    residual = bool(seed % 3 == 0)
+    sep = _run(c, cuda, routed=False, residual=residual)
+    fus = _run(c, cuda, routed=True, residual=residual)
+    routed = (c["se"].cpu() >= start) & (c["se"].cpu() < end)
+    assert float(fus[2][~routed].abs().sum()) == 0.0, tag
+    for name, s, f in zip(NAMES, sep, fus):
+        assert bool(torch.isfinite(f).all()), (name, tag)
+        if float(s.abs().mean()) > 0:
+            assert mean_rel(f, s) <= 1.5e-2, (name, tag, mean_rel(f, s))
+    c["rw"] = torch.ones_like(c["rw"])
+    sep1 = _run(c, cuda, routed=False, residual=residual)
+    fus1 = _run(c, cuda, routed=True, residual=residual)
+    for i in (0, 1, 3, 4, 5):
+        assert torch.equal(sep1[i], fus1[i]), (NAMES[i], tag)
