@@ -47,14 +47,24 @@ enum {
 };
 
 constexpr int BK = 64;  // contraction step, elements
-// shares (in eighths) of a step's direct loads issued after the barrier / with slices 0, 1, 2.
-// Measured on the OLMoE layer: 0/4/4/0 (the A loads behind the first MFMAs of the step, the B loads
-// one slice later) 5.16 ms, 4/4/0/0 5.19, 0/8/0/0 5.31, 0/4/2/2 5.33, 8/0/0/0 5.39, 2/2/2/2 5.53.
+// Shares (in eighths) of a step's direct loads issued after the barrier / with 16-slices 0, 1, 2 of
+// the step.  Forward and input-gradient products (row-major activations): the A loads right after
+// the barrier, the B loads behind the first MFMAs.  Weight gradients (both operands read along the
+// contraction rows): the A loads behind the first MFMAs, the B loads one slice later.  Measured per
+// kernel on one box: the weight gradients gain 4 % with their split and the others lose 1-2 % with
+// it; an even spread over the step, everything in one place, or cutting through the A loads are
+// all 2-7 % worse on the whole layer.
 #ifndef OM_LD_T
-#define OM_LD_T 0
+#define OM_LD_T 4
 #define OM_LD_0 4
-#define OM_LD_1 4
+#define OM_LD_1 0
 #define OM_LD_2 0
+#endif
+#ifndef OM_LDW_T
+#define OM_LDW_T 0
+#define OM_LDW_0 4
+#define OM_LDW_1 4
+#define OM_LDW_2 0
 #endif
 #ifndef OM_ROT_MODE
 #define OM_ROT_MODE 1
@@ -468,9 +478,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // one burst: the texture path of a CU accepts about one 1 KB load per wavefront every ~220
     // cycles, and a wavefront that has to wait for it cannot issue its MFMAs meanwhile.  Shares of
     // the NL loads: after the barrier of step s (stage free), then with slices 0, 1, 2 of step s+1.
-    constexpr int LD_T = NL * OM_LD_T / 8, LD_0 = NL * OM_LD_0 / 8, LD_1 = NL * OM_LD_1 / 8;
+    constexpr bool WG = EPI == EPI_WGRAD;
+    constexpr int LD_T = NL * (WG ? OM_LDW_T : OM_LD_T) / 8, LD_0 = NL * (WG ? OM_LDW_0 : OM_LD_0) / 8;
+    constexpr int LD_1 = NL * (WG ? OM_LDW_1 : OM_LD_1) / 8;
     constexpr int LD_2 = NL - LD_T - LD_0 - LD_1;
-    static_assert(OM_LD_T + OM_LD_0 + OM_LD_1 + OM_LD_2 == 8 && LD_2 >= 0, "load shares");
+    static_assert(OM_LD_T + OM_LD_0 + OM_LD_1 + OM_LD_2 == 8 && OM_LDW_T + OM_LDW_0 + OM_LDW_1 + OM_LDW_2 == 8 &&
+                      LD_2 >= 0, "load shares");
     // wgrad: zero the A c-rows past the end of the expert's rows (after the loads have landed,
     // before the barrier).  B holds finite in-segment data there, so the products vanish.
     auto zero_tail = [&](int step, char *stage) {
