@@ -26,6 +26,12 @@
 //
 // Block order: consecutive block ids go to different XCDs (8 per chip, each with its own L2), so
 // block ids are remapped to give every XCD a contiguous run of tiles, which share operand tiles.
+//
+// Two things that surround the expert GEMMs in the layer are folded into them (template parameters
+// GATHER and ROWW): the token gather (an operand's rows are fetched through an index: the A rows of
+// fwd/dgrad, or the contraction rows of either operand in wgrad), and the routing weight of the
+// combine (the SwiGLU epilogue scales h by the weight of its row; the SwiGLU-backward epilogue
+// scales dh by it and produces the per-row sums that make up the weight's gradient).
 #include "common.h"
 
 namespace {
