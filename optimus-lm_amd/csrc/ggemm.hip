@@ -230,6 +230,54 @@ __device__ __forceinline__ bool find_tile(const int *tile_end, const int *seg, i
     return false;
 }
 
+// Weight gradient: the tiles of expert e cost about (contraction steps of e + a few steps' worth of
+// epilogue) each, so with skewed routing equal tile counts per XCD are far from equal work.  The
+// tiles are numbered expert-major; boundary j of 0..8 is the tile at which j/8 of the launch's work
+// lies behind, and XCD x takes the run [boundary x, boundary x+1).  Every wavefront computes the two
+// boundaries it needs by itself from cum_token_counts (two strided passes, no LDS, no barrier).
+#ifndef OM_WGRAD_EPI_STEPS
+#define OM_WGRAD_EPI_STEPS 3
+#endif
+constexpr int WGRAD_EPILOGUE_STEPS = OM_WGRAD_EPI_STEPS;   // a tile's stores take about as long as 3 steps
+constexpr int WGRAD_BALANCE_MAX_EXPERTS = 4096;
+__device__ __forceinline__ int wgrad_tile_units(int rows, int bk) {
+    const int steps = (rows + bk - 1) / bk;
+    return ((steps + 1) & ~1) + WGRAD_EPILOGUE_STEPS;   // the main loop takes its steps in pairs
+}
+__device__ __forceinline__ void wgrad_xcd_run(const int32_t *cum, int n_experts, int tiles_e, int bk, int xcd,
+                                              int n_xcd, int lane, int &lo, int &hi) {
+    int mine = 0;
+    for (int e = lane; e < n_experts; e += 64) mine += wgrad_tile_units(cum[e + 1] - cum[e], bk);
+    const long long work = static_cast<long long>(wave_sum_i(mine)) * tiles_e;
+    const long long t_lo = work * xcd / n_xcd, t_hi = work * (xcd + 1) / n_xcd;
+    lo = 0;
+    hi = n_experts * tiles_e;
+    int base = 0;   // units of the experts before this chunk
+    for (int e0 = 0; e0 < n_experts; e0 += 64) {
+        const int e = e0 + lane;
+        const int u = e < n_experts ? wgrad_tile_units(cum[e + 1] - cum[e], bk) : 0;
+        int incl = u;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += v;
+        }
+        const long long before = static_cast<long long>(base + incl - u) * tiles_e;
+        const long long after = before + static_cast<long long>(u) * tiles_e;
+        // exactly one expert of the launch holds a target below the total; the total itself
+        // (boundary n_xcd) keeps the initial value of hi
+        const bool has_lo = u > 0 && t_lo >= before && t_lo < after;
+        const bool has_hi = u > 0 && t_hi >= before && t_hi < after;
+        const int tile_lo = e * tiles_e + static_cast<int>((t_lo - before) / (u > 0 ? u : 1));
+        const int tile_hi = e * tiles_e + static_cast<int>((t_hi - before) / (u > 0 ? u : 1));
+        const unsigned long long m_lo = __ballot(has_lo), m_hi = __ballot(has_hi);
+        if (m_lo) lo = __shfl(tile_lo, __ffsll(static_cast<long long>(m_lo)) - 1, 64);
+        if (m_hi) hi = __shfl(tile_hi, __ffsll(static_cast<long long>(m_hi)) - 1, 64);
+        base += __shfl(incl, 63, 64);
+    }
+    if (xcd == 0) lo = 0;
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE,
           bool ROWW = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const GemmParams p) {
@@ -637,14 +685,22 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     }
     const int nbx = gridDim.x / NUM_XCD;
     const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
-    const int per = total_tiles / NUM_XCD, rem = total_tiles - per * NUM_XCD;
+    int per = total_tiles / NUM_XCD, rem = total_tiles - per * NUM_XCD;
+    int run_lo = xcd * per;   // first tile of this XCD's run
+    if (EPI == EPI_WGRAD && p.n_experts <= WGRAD_BALANCE_MAX_EXPERTS) {
+        int lo, hi;
+        wgrad_xcd_run(p.cum, p.n_experts, p.tiles_e, BK, xcd, NUM_XCD, lane, lo, hi);
+        run_lo = __builtin_amdgcn_readfirstlane(lo);
+        per = __builtin_amdgcn_readfirstlane(hi) - run_lo;
+        rem = 0;
+    }
     const int n_mine = slot < per ? (per - slot + nbx - 1) / nbx : 0;
     const int n_all = n_mine + ((xcd < rem && slot == per % nbx) ? 1 : 0);
     int it = 0;
     // moves the per-tile state to this block's next tile that has rows; false when there is none
     auto next_tile = [&]() -> bool {
         while (it < n_all) {
-            const int logical = it < n_mine ? xcd * per + slot + it * nbx : NUM_XCD * per + xcd;
+            const int logical = it < n_mine ? run_lo + slot + it * nbx : total_tiles - rem + xcd;
             it++;
             if (setup_tile(logical)) return true;
         }
