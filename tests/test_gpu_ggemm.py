@@ -27,6 +27,9 @@ def _counts(kind, G, rows, seed=0):
         hot = torch.randperm(G, generator=g)[: max(1, G // 4)]
         c[hot] = rows // len(hot)
         c[hot[0]] += rows - int(c.sum())
+    elif kind == "onehot":   # every row belongs to one expert in the middle
+        c = torch.zeros(G, dtype=torch.long)
+        c[G // 2] = rows
     cum = torch.zeros(G + 1, dtype=torch.int32)
     cum[1:] = torch.cumsum(c, 0)
     return cum
@@ -46,7 +49,10 @@ CASES = [("uniform", 4, 512, 256, 128), ("ragged", 8, 1000, 256, 512), ("empties
          ("ragged", 8, 20000, 512, 768), ("ragged", 8, 20000, 384, 640), ("empties", 32, 9000, 512, 1024),
          # more experts than lanes in a wavefront: the per-block tile table is built in several
          # rounds with a carry, the last one partial
-         ("ragged", 150, 6000, 128, 128), ("empties", 200, 70000, 256, 256)]
+         ("ragged", 150, 6000, 128, 128), ("empties", 200, 70000, 256, 256),
+         # all the work in one expert: the weight gradient's work-balanced split of the tiles over the
+         # XCDs then cuts that expert's tiles eight ways and the zero tiles of the others ride along
+         ("onehot", 70, 5000, 256, 512), ("onehot", 9, 3000, 512, 256), ("onehot", 2, 130, 128, 128)]
 
 
 @pytest.mark.parametrize("kind,G,rows,N,K", CASES)
