@@ -233,13 +233,19 @@ __device__ __forceinline__ bool find_tile(const int *tile_end, const int *seg, i
 // Weight gradient: the tiles of expert e cost about (contraction steps of e + a few steps' worth of
 // epilogue) each, so with skewed routing equal tile counts per XCD are far from equal work.  The
 // tiles are numbered expert-major; boundary j of 0..8 is the tile at which j/8 of the launch's work
-// lies behind, and XCD x takes the run [boundary x, boundary x+1).  Every wavefront computes the two
-// boundaries it needs by itself from cum_token_counts (two strided passes, no LDS, no barrier).
+// lies behind, and XCD x takes the run [boundary x, boundary x+1).  A boundary that falls within an
+// eighth of an XCD's share of an expert's first or last tile moves there: all tiles of dW[g] share
+// the expert's rows of both operands, and with near-uniform routing whole experts per XCD (what
+// equal tile counts give) is the better cut.  Every wavefront computes the two boundaries it needs
+// by itself from cum_token_counts (two strided passes, no LDS, no barrier).
 #ifndef OM_WGRAD_EPI_STEPS
 #define OM_WGRAD_EPI_STEPS 3
 #endif
 constexpr int WGRAD_EPILOGUE_STEPS = OM_WGRAD_EPI_STEPS;   // a tile's stores take about as long as 3 steps
-constexpr int WGRAD_BALANCE_MAX_EXPERTS = 4096;
+#ifndef OM_WGRAD_BALANCE_MAX_EXPERTS
+#define OM_WGRAD_BALANCE_MAX_EXPERTS 4096
+#endif
+constexpr int WGRAD_BALANCE_MAX_EXPERTS = OM_WGRAD_BALANCE_MAX_EXPERTS;
 __device__ __forceinline__ int wgrad_tile_units(int rows, int bk) {
     const int steps = (rows + bk - 1) / bk;
     return ((steps + 1) & ~1) + WGRAD_EPILOGUE_STEPS;   // the main loop takes its steps in pairs
@@ -268,8 +274,16 @@ __device__ __forceinline__ void wgrad_xcd_run(const int32_t *cum, int n_experts,
         // (boundary n_xcd) keeps the initial value of hi
         const bool has_lo = u > 0 && t_lo >= before && t_lo < after;
         const bool has_hi = u > 0 && t_hi >= before && t_hi < after;
-        const int tile_lo = e * tiles_e + static_cast<int>((t_lo - before) / (u > 0 ? u : 1));
-        const int tile_hi = e * tiles_e + static_cast<int>((t_hi - before) / (u > 0 ? u : 1));
+        const long long snap = work / (n_xcd * 8);
+        auto cut = [&](long long t) -> int {   // tile of this expert at which work t lies behind
+            if (t - before <= after - t) {
+                if (t - before <= snap) return e * tiles_e;
+            } else if (after - t <= snap) {
+                return (e + 1) * tiles_e;
+            }
+            return e * tiles_e + static_cast<int>((t - before) / (u > 0 ? u : 1));
+        };
+        const int tile_lo = cut(t_lo), tile_hi = cut(t_hi);
         const unsigned long long m_lo = __ballot(has_lo), m_hi = __ballot(has_hi);
         if (m_lo) lo = __shfl(tile_lo, __ffsll(static_cast<long long>(m_lo)) - 1, 64);
         if (m_hi) hi = __shfl(tile_hi, __ffsll(static_cast<long long>(m_hi)) - 1, 64);
