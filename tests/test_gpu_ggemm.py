@@ -289,3 +289,29 @@ def test_gathered_merged_mlp_random_shapes(cuda, seed):
         results.append([y.detach(), xd.grad] + [w.grad for w in wd])
     for name, a, b in zip(("y", "dx", "dw_gate", "dw_up", "dw_down"), *results):
         assert torch.equal(a, b), (name, T, K, N, start, end, I, H)
+
+
+@pytest.mark.parametrize("G,rows,N,K", [(4096, 9000, 128, 256), (4097, 9000, 256, 128), (5000, 6000, 128, 128)])
+def test_wgrad_with_thousands_of_experts(cuda, G, rows, N, K):
+    """The weight gradient has no limit on the number of experts (the forward/dgrad tile table has).
+    Up to 4096 experts its tiles are split over the XCDs by estimated work, above that by count:
+    both sides of that threshold, most experts with 0-3 rows, against per-expert fp32 matmul."""
+    from optimus import _native as n
+    g = torch.Generator().manual_seed(G)
+    c = torch.bincount(torch.randint(0, G, (rows,), generator=g), minlength=G)
+    cum = torch.zeros(G + 1, dtype=torch.int32)
+    cum[1:] = torch.cumsum(c, 0)
+    dy = torch.randn(rows, N, generator=g).to(torch.bfloat16)
+    x = torch.randn(rows, K, generator=g).to(torch.bfloat16)
+    dyd, xd, cumd = dy.to(cuda), x.to(cuda), cum.to(cuda)
+    dw = torch.full((G, N, K), float("nan"), dtype=torch.bfloat16, device=cuda)
+    n.check(n.lib().om_grouped_gemm_wgrad(n.ptr(dyd), n.ptr(xd), n.ptr(dw), n.ptr(cumd), rows, G, N, K, 0,
+                                          n.stream()), "om_grouped_gemm_wgrad")
+    got = dw.float().cpu()
+    assert bool(torch.isfinite(got).all())      # every tile of every expert was written
+    ref = torch.zeros(G, N, K)
+    for e in torch.nonzero(c).flatten().tolist():
+        s, t = int(cum[e]), int(cum[e + 1])
+        ref[e] = dy[s:t].float().t() @ x[s:t].float()
+    assert max_abs(got, ref) <= 1e-2 * max(1.0, float(ref.abs().max()))
+    assert float(got[c == 0].abs().max()) == 0.0
