@@ -52,8 +52,10 @@ def moe_inputs(name, dtype=torch.bfloat16, scale_tokens=1.0):
     return out
 
 
-def dsv3_inputs(dtype=torch.bfloat16, scale_tokens=1.0, scale_hidden=1.0):
+def dsv3_inputs(dtype=torch.bfloat16, scale_tokens=1.0, scale_hidden=1.0, seed=None):
     cfg = dict(DSV3_SHAPE)
+    if seed is not None:
+        cfg["seed"] = seed
     cfg["T"] = max(8, int(cfg["T"] * scale_tokens) // 8 * 8)
     cfg["H"] = max(128, int(cfg["H"] * scale_hidden) // 128 * 128)
     cfg["I"] = max(128, int(cfg["I"] * scale_hidden) // 128 * 128)

@@ -57,6 +57,23 @@ def dsv3_topk_indices(scores, bias, n_group, topk_group, top_k):
     return _topk_stable(scores_for_choice, top_k)[1], scores_for_choice               # :179
 
 
+def dsv3_selection_margin(scores, bias, n_group, topk_group, top_k):
+    """Per token, the smallest gap that the group-limited selection (modeling_deepseek_v3.py:164-180)
+    rests on: between the last kept and the first dropped group score, and between the K-th and
+    the (K+1)-th choice value among the kept groups.  A fixture whose margins all exceed the
+    difference two fp32 evaluations of the logits can have (summation order: ~1e-7) selects the
+    same expert SETS on the CPU and the GPU, which is what makes set-exact parity a fair demand."""
+    T, N = scores.shape
+    choice = scores.view(-1, N) + bias.unsqueeze(0)
+    group_scores = _topk_stable(choice.view(-1, n_group, N // n_group), 2)[0].sum(dim=-1)
+    gs = torch.sort(group_scores, dim=-1, descending=True).values
+    group_gap = gs[:, topk_group - 1] - gs[:, topk_group] if topk_group < n_group else torch.full((T,), float("inf"))
+    _, masked = dsv3_topk_indices(scores, bias, n_group, topk_group, top_k)
+    ms = torch.sort(masked, dim=-1, descending=True).values
+    choice_gap = ms[:, top_k - 1] - ms[:, top_k]
+    return torch.minimum(group_gap, choice_gap)
+
+
 def dsv3_router(hidden_states, weight, bias, n_group, topk_group, top_k, norm_topk_prob,
                 routed_scaling_factor):
     """-> (topk_indices [T,K] int64, topk_weights [T,K] fp32, router_logits fp32)."""

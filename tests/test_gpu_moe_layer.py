@@ -1,8 +1,13 @@
 """Whole-layer parity of the MoE modules against the fp32 restatement of the reference blocks.
 
-Bar (north star): expert indices bit-exact; outputs and gradients max-abs <= 2e-2 and mean-rel
-<= 1e-3 against the fp32 reference evaluated on the same bf16-rounded inputs (mean_rel :=
-mean|a-b| / mean|b|)."""
+Bar: expert indices bit-exact; outputs and gradients max-abs <= 2e-2 (times the reference's largest
+magnitude where that exceeds 1) against the fp32 reference evaluated on the same bf16-rounded
+inputs.  The mean-rel bar (mean_rel := mean|a-b| / mean|b|) is stated as an excess over an ideally
+rounded oracle: one bf16 rounding of the fp32 reference itself already has mean_rel 1.41e-3, so a
+flat 1e-3 cannot be met by any bf16 result.  util.assert_bf16_parity holds
+mean_rel(gpu, ref) <= excess * mean_rel(bf16(ref), ref) and an absolute cap close to the measured
+figure; the layer keeps g, u, h and y in bf16 like the reference, which is where the 2-3 roundings'
+worth of excess comes from.  LAYER_BARS lists (excess, cap) per tensor."""
 import numpy as np
 import pytest
 import torch
@@ -10,11 +15,15 @@ import torch
 import synthetic_configs as sc
 from oracle import moe_layer as L
 from oracle import routing as R
-from util import max_abs, mean_rel
+from util import assert_bf16_parity, max_abs, mean_rel
 
 pytestmark = pytest.mark.gpu
 
-MAX_ABS, MEAN_REL = 2e-2, 1e-3
+MAX_ABS = 2e-2
+# (excess over the bf16 floor, absolute cap on mean_rel) for the layer's output and its gradients
+LAYER_BARS = {"out": (6.0, 1e-2), "grad": (6.0, 1e-2)}
+ODD_BARS = {"out": (6.0, 1e-2), "grad": (8.0, 1.5e-2)}
+DSV3_GATE_BAR = (12.0, 2e-2)
 
 
 def _olmoe_block(inp, cuda, fast=True, merged=True, fp32_logits=True):
@@ -72,14 +81,13 @@ def test_fast_block_fwd_bwd(cuda, name, scale):
     _, e_gpu, _ = R.olmoe_router(logits.float().cpu(), c["K"], c["norm_topk_prob"], torch.float32)
     assert torch.equal(e_ref, e_gpu)
     o = out.float().cpu().view(c["T"], c["H"])
-    assert max_abs(o, ref_out) <= MAX_ABS and mean_rel(o, ref_out) <= 4e-3, (max_abs(o, ref_out), mean_rel(o, ref_out))
+    assert_bf16_parity(o, ref_out, *LAYER_BARS["out"], tag=f"fast_block[{name}] out", max_abs_bar=MAX_ABS)
     got = {"x": x.grad.view(c["T"], c["H"]), "gate_w": blk.gate.weight.grad,
            "w_gate": blk.experts.gate_proj_merged_weight.grad, "w_up": blk.experts.up_proj_merged_weight.grad,
            "w_down": blk.experts.down_proj_merged_weight.grad}
     for k, gref in ref_grads.items():
-        a = got[k].float().cpu()
-        assert mean_rel(a, gref) <= 1e-2, (k, mean_rel(a, gref))
-        assert max_abs(a, gref) <= MAX_ABS * max(1.0, float(gref.abs().max())), (k, max_abs(a, gref))
+        assert_bf16_parity(got[k], gref, *LAYER_BARS["grad"], tag=f"fast_block[{name}] d{k}",
+                           max_abs_bar=MAX_ABS * max(1.0, float(gref.abs().max())))
 
 
 @pytest.mark.parametrize("T,H,I,N,K,renorm", [
@@ -111,14 +119,15 @@ def test_fast_block_odd_small_shapes(cuda, T, H, I, N, K, renorm):
     _, e_gpu, _ = R.olmoe_router(logits.float().cpu(), K, renorm, torch.float32)
     assert torch.equal(e_ref, e_gpu)
     o = out.detach().float().cpu().view(T, H)
-    assert max_abs(o, ref_out) <= MAX_ABS * max(1.0, float(ref_out.abs().max())) and mean_rel(o, ref_out) <= 6e-3
+    tag = f"odd[{T},{H},{I},{N},{K}]"
+    assert_bf16_parity(o, ref_out, *ODD_BARS["out"], tag=tag + " out",
+                       max_abs_bar=MAX_ABS * max(1.0, float(ref_out.abs().max())))
     got = {"x": x.grad.view(T, H), "gate_w": blk.gate.weight.grad,
            "w_gate": blk.experts.gate_proj_merged_weight.grad, "w_up": blk.experts.up_proj_merged_weight.grad,
            "w_down": blk.experts.down_proj_merged_weight.grad}
     for k, gref in ref_grads.items():
-        a = got[k].float().cpu()
-        assert mean_rel(a, gref) <= 1.5e-2, (k, mean_rel(a, gref))
-        assert max_abs(a, gref) <= MAX_ABS * max(1.0, float(gref.abs().max())), (k, max_abs(a, gref))
+        assert_bf16_parity(got[k], gref, *ODD_BARS["grad"], tag=f"{tag} d{k}",
+                           max_abs_bar=MAX_ABS * max(1.0, float(gref.abs().max())))
 
 
 @pytest.mark.parametrize("merged", [True, False])
@@ -171,10 +180,14 @@ def test_fast_block_float32_c1(cuda, merged):
         assert max_abs(a, gref) <= 1e-4 * max(1.0, float(gref.abs().max())), (k, max_abs(a, gref))
 
 
-def test_fast_block_injected_logits_skewed(cuda):
+@pytest.mark.parametrize("path", ["separate", "fused"])
+def test_fast_block_injected_logits_skewed(cuda, path):
     """C4: Zipf-skewed routing injected at the functional level (router logits given): many experts
-    get 0-8 rows, a few get hundreds.  Expert computation only (router excluded), fwd+bwd."""
-    from optimus.models.common.moe import SoftmaxTopkRouterFunction, MergedMLPFunction, expert_computation
+    get 0-8 rows, a few get hundreds.  Expert computation only (router excluded), fwd+bwd, both as
+    the reference's sequence of separate functions (K4, MergedMLP, K6) and as the blocks' default
+    (RoutedMLPFunction: gather and routing weight inside the expert GEMMs), each against fp32."""
+    from optimus.models.common.moe import (SoftmaxTopkRouterFunction, MergedMLPFunction, RoutedMLPFunction,
+                                           expert_computation)
     inp = sc.moe_inputs("C4")
     c = inp["cfg"]
     logits = inp["logits"]
@@ -187,7 +200,11 @@ def test_fast_block_injected_logits_skewed(cuda):
     t = {k: inp[k].to(cuda).requires_grad_(True) for k in ("x", "w_gate", "w_up", "w_down")}
     wd = w.detach().requires_grad_(True)
     fn = lambda gi, cum: MergedMLPFunction.apply(gi, t["w_gate"], t["w_up"], t["w_down"], cum)
-    out = expert_computation(t["x"], wd, e, 0, c["N"], fn, c["N"])
+    routed = None
+    if path == "fused":
+        routed = lambda hs, rw, ii, cum_ep, oi, si, cum, res: RoutedMLPFunction.apply(
+            hs, rw, ii, cum_ep, oi, si, cum, res, True, t["w_gate"], t["w_up"], t["w_down"])
+    out = expert_computation(t["x"], wd, e, 0, c["N"], fn, c["N"], routed_experts_fn=routed)
     out.backward(inp["dout"].to(cuda))
     r = {k: inp[k].float().requires_grad_(True) for k in ("x", "w_gate", "w_up", "w_down")}
     wr = w_ref.float().requires_grad_(True)
@@ -197,10 +214,10 @@ def test_fast_block_injected_logits_skewed(cuda):
         if tok.numel():
             ref = ref.index_add(0, tok, L.expert_mlp(r["x"][tok], r["w_gate"][n], r["w_up"][n], r["w_down"][n]) * wr[tok, kk, None])
     ref.backward(inp["dout"].float())
-    assert max_abs(out.float().cpu(), ref.detach()) <= MAX_ABS and mean_rel(out.float().cpu(), ref.detach()) <= 4e-3
+    assert_bf16_parity(out, ref, *LAYER_BARS["out"], tag=f"C4[{path}] out", max_abs_bar=MAX_ABS)
     for k in r:
-        assert mean_rel(t[k].grad.float().cpu(), r[k].grad) <= 1e-2, k
-    assert mean_rel(wd.grad.float().cpu(), wr.grad) <= 1e-2
+        assert_bf16_parity(t[k].grad, r[k].grad, *LAYER_BARS["grad"], tag=f"C4[{path}] d{k}")
+    assert_bf16_parity(wd.grad, wr.grad, *LAYER_BARS["grad"], tag=f"C4[{path}] d routing_weights")
     empty = counts == 0
     if empty.any():
         assert float(t["w_gate"].grad[empty.to(cuda)].abs().max()) == 0.0
@@ -344,14 +361,31 @@ def test_block_with_residual_equals_block_plus_add(cuda):
     assert torch.equal(results[0][2], inp["dout"].to(cuda).view_as(results[0][2]))
 
 
+def _dsv3_fixture(scale_tokens, scale_hidden, margin=2e-6):
+    """The seeded C5 inputs at a reduced size, with the seed advanced until every token's selection
+    margin (oracle.routing.dsv3_selection_margin, evaluated in float64) exceeds `margin`: two fp32
+    evaluations of the 7168-term (here shorter) logit sums differ by ~1e-7 in the scores, so with
+    this margin the CPU restatement and the GPU select the same expert sets for EVERY token."""
+    for seed in range(sc.DSV3_SHAPE["seed"], sc.DSV3_SHAPE["seed"] + 16):
+        inp = sc.dsv3_inputs(scale_tokens=scale_tokens, scale_hidden=scale_hidden, seed=seed)
+        c = inp["cfg"]
+        scores = torch.sigmoid(inp["x"].double() @ inp["router_w"].to(torch.bfloat16).double().t())
+        m = R.dsv3_selection_margin(scores, inp["bias"].double(), c["n_group"], c["topk_group"], c["K"])
+        if float(m.min()) > margin:
+            return inp
+    raise AssertionError("no seed with a safe selection margin in 16 tries")
+
+
 @pytest.mark.parametrize("ep_ind", [0, 3])
 def test_dsv3_block_one_rank_share(cuda, ep_ind):
     """C5 at reduced size: DeepseekV3ParallelMoE with expert_parallelism=8 (32 of 256 routed experts
-    local) + shared expert, against the fp32 restatement of the reference block."""
+    local) + shared expert, against the fp32 restatement of the reference block (pinned on the CPU
+    by tests/test_oracle_moe.py::test_dsv3_block_*).  The fixture has a safe selection margin, so the
+    expert sets of all tokens must agree and every gradient is compared unconditionally."""
     from optimus.mapper import ParallelDpPpEpTpMapper
     from optimus.models.deepseek_v3.configuration_deepseek_v3 import DeepseekV3ParallelConfig
     from optimus.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3ParallelMoE
-    inp = sc.dsv3_inputs(scale_tokens=1 / 16, scale_hidden=1 / 7)
+    inp = _dsv3_fixture(1 / 16, 1 / 7)
     c = inp["cfg"]
     cfg = DeepseekV3ParallelConfig(hidden_size=c["H"], moe_intermediate_size=c["I"], n_routed_experts=c["N"],
                                    n_group=c["n_group"], topk_group=c["topk_group"], num_experts_per_tok=c["K"],
@@ -372,6 +406,7 @@ def test_dsv3_block_one_rank_share(cuda, ep_ind):
     out.backward(inp["dout"].to(cuda).view_as(out))
     # reference in fp32 on the same (bf16-rounded) values; router weight as the module holds it
     rw = blk.gate.weight.detach().float().cpu()
+    assert torch.equal(rw, inp["router_w"].to(torch.bfloat16).float())
     names = ("x", "w_gate", "w_up", "w_down", "ws_gate", "ws_up", "ws_down")
     t = {k: inp[k].float().requires_grad_(True) for k in names}
     rwt = rw.clone().requires_grad_(True)
@@ -380,15 +415,21 @@ def test_dsv3_block_one_rank_share(cuda, ep_ind):
                                          t["ws_up"], t["ws_down"], c["n_group"], c["topk_group"], c["K"], True, 2.5,
                                          expert_start_idx=ep_ind * c["NR"])
     ref.backward(inp["dout"].float())
-    # routing: same expert sets per token (the reference leaves the order unspecified)
-    e_gpu, _ = blk.gate(x.detach())
-    same = (torch.sort(e_gpu.cpu(), 1).values == torch.sort(e_ref, 1).values).all(1)
-    assert float(same.float().mean()) >= 0.999       # fp32 GEMM summation order can flip a near-tie
-    o = out.float().cpu().view(c["T"], c["H"])[same]
-    assert max_abs(o, ref.detach()[same]) <= MAX_ABS and mean_rel(o, ref.detach()[same]) <= 4e-3
-    if bool(same.all()):
-        assert mean_rel(x.grad.float().cpu().view(c["T"], c["H"]), t["x"].grad) <= 1e-2
-        assert mean_rel(blk.shared_experts.up_proj.weight.grad.float().cpu(), t["ws_up"].grad) <= 1e-2
-        got = torch.stack([m.down_proj.weight.grad for m in blk.experts]).float().cpu()
-        assert mean_rel(got, t["w_down"].grad) <= 1e-2
-        assert mean_rel(blk.gate.weight.grad.float().cpu(), rwt.grad) <= 2e-2
+    # routing: same expert sets for every token (the reference leaves the order unspecified)
+    e_gpu, w_gpu = blk.gate(x.detach())
+    assert torch.equal(torch.sort(e_gpu.cpu(), 1).values, torch.sort(e_ref, 1).values)
+    order_g, order_r = torch.argsort(e_gpu.cpu(), 1), torch.argsort(e_ref, 1)
+    assert torch.allclose(w_gpu.float().cpu().gather(1, order_g), w_ref.detach().gather(1, order_r), rtol=2e-5, atol=1e-7)
+    local = (e_ref >= ep_ind * c["NR"]) & (e_ref < (ep_ind + 1) * c["NR"])
+    assert int(local.sum()) > 0.5 * c["T"]             # the window really gets about T routed rows
+    tag = f"dsv3_share[{ep_ind}]"
+    o = out.float().cpu().view(c["T"], c["H"])
+    assert_bf16_parity(o, ref, *LAYER_BARS["out"], tag=tag + " out", max_abs_bar=MAX_ABS)
+    assert_bf16_parity(x.grad.view(c["T"], c["H"]), t["x"].grad, *LAYER_BARS["grad"], tag=tag + " dx")
+    stack = lambda attr: torch.stack([getattr(m, attr).weight.grad for m in blk.experts])
+    for attr, key in (("gate_proj", "w_gate"), ("up_proj", "w_up"), ("down_proj", "w_down")):
+        assert_bf16_parity(stack(attr), t[key].grad, *LAYER_BARS["grad"], tag=f"{tag} d{key}")
+        assert_bf16_parity(getattr(blk.shared_experts, attr).weight.grad, t["ws" + key[1:]].grad,
+                           *LAYER_BARS["grad"], tag=f"{tag} dws{key[1:]}")
+    # the router weight gets its gradient only through the K gathered scores of each token
+    assert_bf16_parity(blk.gate.weight.grad, rwt.grad, *DSV3_GATE_BAR, tag=tag + " drouter_w")

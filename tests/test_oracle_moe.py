@@ -172,3 +172,112 @@ def test_layer_restatements_agree_on_tiny_shapes():
         f, _ = L.fast_block_restatement(x, w, e, wg[s:s + 4], wu[s:s + 4], wd[s:s + 4], expert_start_idx=s)
         parts.append(f)
     assert torch.allclose(parts[0] + parts[1], fast, atol=1e-5)
+
+
+def _dsv3_tiny(seed=3):
+    """A DeepSeek-V3-shaped toy: 16 experts in 4 groups, 2 groups kept, top-4, one shared expert."""
+    g = torch.Generator().manual_seed(seed)
+    T, H, N, I = 40, 24, 16, 20
+    x = torch.randn(T, H, generator=g)
+    Wr = torch.randn(N, H, generator=g) * 0.3
+    bias = torch.randn(N, generator=g) * 0.1
+    wg = torch.randn(N, I, H, generator=g) * 0.2
+    wu = torch.randn(N, I, H, generator=g) * 0.2
+    wd = torch.randn(N, H, I, generator=g) * 0.2
+    sg = torch.randn(I, H, generator=g) * 0.2
+    su = torch.randn(I, H, generator=g) * 0.2
+    sd = torch.randn(H, I, generator=g) * 0.2
+    return dict(x=x, Wr=Wr, bias=bias, wg=wg, wu=wu, wd=wd, sg=sg, su=su, sd=sd,
+                route=dict(n_group=4, topk_group=2, top_k=4, norm_topk_prob=True,
+                           routed_scaling_factor=2.5))
+
+
+def _dsv3_block(c, start=0, count=None, shared=True, tensors=None):
+    from oracle import moe_layer as L
+    t = tensors or c
+    count = c["wg"].shape[0] if count is None else count
+    sl = slice(start, start + count)
+    zero = torch.zeros_like
+    ws = (t["sg"], t["su"], t["sd"]) if shared else (zero(t["sg"]), zero(t["su"]), zero(t["sd"]))
+    return L.dsv3_moe_block(t["x"], t["Wr"], t["bias"], t["wg"][sl], t["wu"][sl], t["wd"][sl], *ws,
+                            expert_start_idx=start, **c["route"])
+
+
+def test_dsv3_block_is_dense_formula_plus_shared_expert():
+    """Pins oracle.moe_layer.dsv3_moe_block (modeling_deepseek_v3.py:221-275) on a tiny shape against
+    evaluations that share none of its code: the token-by-token textbook sum over the routed experts
+    (weights and ids from the brute-force-pinned router) plus the shared expert's MLP on every
+    token.  Deliberately wrong variants (no shared expert, a window offset by one expert, weights
+    taken from the biased scores) must fail the same comparison."""
+    from oracle import moe_layer as L, routing as R
+    c = _dsv3_tiny()
+    out, ids, w = _dsv3_block(c)
+    ids_r, w_r, _ = R.dsv3_router(c["x"], c["Wr"], c["bias"], **c["route"])
+    assert torch.equal(ids, ids_r) and torch.equal(w, w_r)
+    # router invariants that fix its meaning: K distinct experts, from at most topk_group groups,
+    # weights sum to the scaling factor
+    assert all(len(set(r.tolist())) == 4 for r in ids)
+    assert all(len({int(e) // 4 for e in r}) <= 2 for r in ids)
+    assert torch.allclose(w.sum(1), torch.full((w.shape[0],), 2.5), atol=1e-5)
+    routed = L.dense_formula(c["x"], w, ids, c["wg"], c["wu"], c["wd"])
+    shared = L.expert_mlp(c["x"], c["sg"], c["su"], c["sd"])
+    assert torch.allclose(out, routed + shared, atol=2e-5)
+    scale = float(out.abs().mean())
+    # a block without its shared expert is a different function
+    assert float((out - routed).abs().mean()) > 0.05 * scale
+    # so is one whose window is offset by one expert (weights of expert e+1 used for id e) ...
+    shifted = L.dense_formula(c["x"], w, ids, c["wg"].roll(1, 0), c["wu"].roll(1, 0), c["wd"].roll(1, 0))
+    assert float((out - shifted - shared).abs().mean()) > 0.05 * scale
+    # ... and one whose weights come from sigmoid + bias instead of the plain sigmoid (:187)
+    s = torch.sigmoid(torch.nn.functional.linear(c["x"], c["Wr"]))
+    wb = (s + c["bias"]).gather(1, ids)
+    wb = wb / (wb.sum(1, keepdim=True) + 1e-20) * 2.5
+    biased = L.dense_formula(c["x"], wb, ids, c["wg"], c["wu"], c["wd"])
+    assert float((out - biased - shared).abs().mean()) > 1e-3 * scale
+
+
+def test_dsv3_block_windows_sum_to_the_whole_block():
+    """Expert parallelism of the DeepSeek-V3 block (modeling_deepseek_v3.py:226-229): each rank adds
+    only its window's experts, so the routed parts of all ranks' blocks sum to the EP=1 routed part,
+    and a window that owns no selected expert contributes exactly the shared expert."""
+    from oracle import moe_layer as L
+    c = _dsv3_tiny(seed=4)
+    full, ids, _ = _dsv3_block(c, shared=False)
+    parts = [_dsv3_block(c, start=s, count=4, shared=False)[0] for s in (0, 4, 8, 12)]
+    assert torch.allclose(sum(parts), full, atol=2e-5)
+    # every window is a strict part (none is empty, none is everything) for this fixture
+    assert all(0.0 < float(p.abs().sum()) < float(full.abs().sum()) for p in parts)
+    # a window's block only sees tokens that chose one of its experts
+    for s, p in zip((0, 4, 8, 12), parts):
+        hit = ((ids >= s) & (ids < s + 4)).any(1)
+        assert torch.equal(p[~hit], torch.zeros_like(p[~hit]))
+        assert bool((p[hit].abs().sum(1) > 0).all())
+    with_shared = _dsv3_block(c, start=4, count=4, shared=True)[0]
+    assert torch.allclose(with_shared - parts[1], L.expert_mlp(c["x"], c["sg"], c["su"], c["sd"]), atol=2e-5)
+
+
+def test_dsv3_block_gradients_match_the_dense_formula():
+    """Backward of the DeepSeek-V3 block restatement: autograd through the per-expert index_add_
+    loop against autograd through the token-by-token formula (separate graphs), for the input,
+    the router weight (reached only through the gathered sigmoid scores: the index selection is
+    no_grad and the bias gets no gradient, modeling_deepseek_v3.py:186-187) and the experts."""
+    from oracle import moe_layer as L, routing as R
+    c = _dsv3_tiny(seed=5)
+    names = ("x", "Wr", "wg", "wu", "wd", "sg", "su", "sd")
+    d = torch.randn(c["x"].shape, generator=torch.Generator().manual_seed(9))
+
+    a = {k: (v.clone().requires_grad_(True) if k in names else v) for k, v in c.items()}
+    a["bias"] = c["bias"].clone().requires_grad_(True)
+    out, ids, w = _dsv3_block(c, tensors=a)
+    out.backward(d)
+    assert a["bias"].grad is None
+
+    b = {k: (v.clone().requires_grad_(True) if k in names else v) for k, v in c.items()}
+    ids_b, w_b, _ = R.dsv3_router(b["x"], b["Wr"], b["bias"], **c["route"])
+    ref = L.dense_formula(b["x"], w_b, ids_b, b["wg"], b["wu"], b["wd"]) + \
+        L.expert_mlp(b["x"], b["sg"], b["su"], b["sd"])
+    ref.backward(d)
+    for k in names:
+        assert torch.allclose(a[k].grad, b[k].grad, rtol=1e-4, atol=1e-5), k
+    # the routing weights do carry gradient into the router weight
+    assert float(a["Wr"].grad.abs().sum()) > 0
