@@ -86,6 +86,12 @@ int om_grad_norm_clip_coef(const float *partials, const int64_t *seg_first_chunk
                            int64_t n_segs, int grad_dtype, double max_norm, float *seg_norms,
                            float *total_norm, float *clip_coef, void *stream);
 
+/* om_grad_scale: grad = cast(float(grad) * *coef) in place over n elements, coef a device fp32
+ * scalar (the clip_coef above): the in-place multiply of clip_grads_with_norm_
+ * (optimizers.py:145/150/154) for gradient tensors that no update kernel reads (parameters of the
+ * model that the optimizer does not hold, or skip_optimizer_step).  grad 16-byte aligned.       */
+int om_grad_scale(void *grad, int64_t n, int grad_dtype, const float *coef, void *stream);
+
 /* om_adamw_step with the clip folded in: g = cast(grad * *grad_scale) is what the update uses,
  * i.e. the in-place multiply of clip_grads_with_norm_ (optimizers.py:145/150/154) without its
  * read-modify-write pass over the gradients.  *grad_scale is a device fp32 scalar (the clip_coef

@@ -127,7 +127,49 @@ __global__ __launch_bounds__(256) void total_norm_kernel(const float *__restrict
     }
 }
 
+// grad = cast(float(grad) * *coef), 16 bytes per lane, scalar tail.
+template <typename T>
+__global__ __launch_bounds__(256) void grad_scale_kernel(T *__restrict__ grad, int64_t n,
+                                                         const float *__restrict__ coef) {
+    constexpr int V = Elem<T>::VEC;
+    const float c = *coef;
+    const int64_t nv = n / V;
+    u32x4 *vp = reinterpret_cast<u32x4 *>(grad);
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t j = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; j < nv; j += stride) {
+        float f[V];
+        Elem<T>::unpack(vp[j], f);
+#pragma unroll
+        for (int i = 0; i < V; i++) f[i] = f[i] * c;
+        vp[j] = Elem<T>::pack(f);
+    }
+    if (blockIdx.x == 0) {
+        const int64_t i = nv * V + threadIdx.x;
+        if (i < n) Elem<T>::store(grad + i, Elem<T>::load(grad + i) * c);
+    }
+}
+
 }  // namespace
+
+extern "C" int om_grad_scale(void *grad, int64_t n, int grad_dtype, const float *coef, void *stream) {
+    if (grad_dtype != OM_BF16 && grad_dtype != OM_F32) return OM_ERR_DTYPE;
+    if (n < 0) return OM_ERR_SHAPE;
+    if (n == 0) return OM_OK;
+    if (!grad || !coef) return OM_ERR_NULL;
+    if (!om_aligned16(grad)) return OM_ERR_ALIGN;
+    const int vec = grad_dtype == OM_BF16 ? 8 : 4;
+    int64_t blocks = (n / vec + 255) / 256;
+    if (blocks < 1) blocks = 1;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    hipStream_t st = om_stream(stream);
+    if (grad_dtype == OM_BF16)
+        grad_scale_kernel<uint16_t><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(
+            static_cast<uint16_t *>(grad), n, coef);
+    else
+        grad_scale_kernel<float><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(
+            static_cast<float *>(grad), n, coef);
+    return om_launch_status();
+}
 
 extern "C" int om_grad_sumsq(const void *grad, int grad_dtype, const int64_t *chunk_offsets,
                              int64_t n_chunks, float *partials, void *stream) {

@@ -13,14 +13,18 @@ from optimus import _native as _n
 from optimus.profilers import record_pcl_function
 
 
+_STATE_KEYS = ("flat_exp_avg", "flat_exp_avg_sq", "flat_fp32_master_param")
+
+
 class MixedPrecisionAdamW(Optimizer):
-    """
-    Stores all parameters, gradients, and optimizer states into a flat buffer.
-    Optimizer states include exp_avg and exp_avg_sq which are in FP32
-    Master weights are stored in FP32
-    ## Limitations
-    1. Only one param group
-    2. One GPU: num_shards must be 1 (the data-parallel all-reduce is outside this build)
+    """AdamW over five flat buffers, interface of the reference class (optimus/optimizers.py:19-225).
+
+    `flat_param` / `flat_grad` hold every parameter and gradient in the model dtype, back to back in
+    `param_list` order; `flat_exp_avg`, `flat_exp_avg_sq`, `flat_fp32_master_param` are float32.  After
+    construction each `p.data` and `p.grad` is a view of its slice, so backward accumulates straight
+    into the buffer the update kernel reads.  In float32 mode the master weights are `flat_param`
+    itself.  Constraints kept from the reference: one parameter group, `device` given, no expert
+    parallelism; beyond it: one GPU (`num_shards == 1`, no tensor parallelism), float32 or bfloat16.
     """
 
     def __init__(self,
@@ -39,150 +43,133 @@ class MixedPrecisionAdamW(Optimizer):
                  expert_parallelism=1, ep_ind=0, ep_group=None,
                  dpep_ind=0, dpep_group=None,
                  skip_optimizer_step=False):
-        defaults = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay)
-        super().__init__(params, defaults)
-
-        assert device is not None
+        super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
+        if device is None:
+            raise AssertionError("MixedPrecisionAdamW needs the device of the flat buffers")
         if dtype not in (torch.float32, torch.bfloat16):
             raise TypeError("MixedPrecisionAdamW: dtype must be torch.float32 or torch.bfloat16")
-
-        self.model = model
-        self.warmup_steps = warmup_steps
-        self.dtype = dtype
-        self.device = device
-        self.opt_disable_delayed_grad_clipping = opt_disable_delayed_grad_clipping
-        self.opt_use_two_step_grad_clipping = opt_use_two_step_grad_clipping
-        self.opt_use_chunked_allreduce = opt_use_chunked_allreduce
-        self.profiler = profiler
-
-        self.tensor_parallelism = tensor_parallelism
-        self.tp_ind = tp_ind
-        self.tp_group = tp_group
-
-        self.expert_parallelism = expert_parallelism
-        self.ep_ind = ep_ind
-        self.ep_group = ep_group
-
-        assert self.expert_parallelism == 1, "This optimizer does not support expert parallelism."
-        assert self.tensor_parallelism == 1, "tensor parallelism is outside the single-GPU hot path"
-
-        self.dpep_ind = dpep_ind
-        self.dpep_group = dpep_group
-        self.skip_optimizer_step = skip_optimizer_step
-
-        self.step_id = 0
-
-        # Sharding options (reference optimizers.py:73-76); one GPU here
+        if len(self.param_groups) != 1:
+            raise AssertionError("Only one parameter group is supported")
+        if expert_parallelism != 1:
+            raise AssertionError("This optimizer does not support expert parallelism.")
+        if tensor_parallelism != 1:
+            raise AssertionError("tensor parallelism is outside the single-GPU hot path")
         if num_shards != 1:
             raise NotImplementedError("num_shards > 1 (data-parallel all-reduce) is not part of "
                                       "the single-GPU hot path")
-        self.num_shards = num_shards
-        self.dp_ind = shard_id
-        self.group = group
-
-        self.param_list = [p for pg in self.param_groups for p in pg["params"]]
-        assert len([pg for pg in self.param_groups]) == 1, "Only one parameter group is supported"
-
-        self.param_sizes = [p.numel() for p in self.param_list]
-        self.param_start_inds = [sum(self.param_sizes[0:i]) for i in range(len(self.param_sizes))]
-        self.flat_param_size = sum(self.param_sizes)
-
-        # Flat buffers
-        self.flat_param = torch.empty(self.flat_param_size, dtype=self.dtype, device=self.device)
-        self.flat_grad = torch.zeros(self.flat_param_size, dtype=self.dtype, device=self.device)
-        if not self.skip_optimizer_step:
-            self.flat_exp_avg = torch.zeros(self.flat_param_size, dtype=torch.float32, device=self.device)
-            self.flat_exp_avg_sq = torch.zeros(self.flat_param_size, dtype=torch.float32, device=self.device)
-        else:
-            self.flat_exp_avg = None
-            self.flat_exp_avg_sq = None
-
-        if self.dtype != torch.float32:
-            if not self.skip_optimizer_step:
-                self.flat_fp32_master_param = torch.zeros(self.flat_param_size, dtype=torch.float32,
-                                                          device=self.device)
-            else:
-                self.flat_fp32_master_param = None
-        else:
-            # FP32 optimizer: master param and model param share one buffer
-            self.flat_fp32_master_param = self.flat_param
-
-        # Mapping parameter into flat parameter.
-        for param_id, p in enumerate(self.param_list):
-            start_ind = self.param_start_inds[param_id]
-            end_ind = self.param_start_inds[param_id] + self.param_sizes[param_id]
-            p.data = self.flat_param[start_ind:end_ind].view_as(p.data).copy_(p.data)
-            p.grad = self.flat_grad[start_ind:end_ind].view_as(p.data)
-            if self.dtype != torch.float32 and (not self.skip_optimizer_step):
-                self.flat_fp32_master_param[start_ind:end_ind].view_as(p.data).copy_(p.data)
-
-        # Gradient-norm kernels run over flat_grad when it holds every gradient of the model
-        # (the reference takes the norm over model.parameters(), optimizers.py:143-158)
+        # attributes the training driver and the sharded variants of the reference read
+        for name, value in (("model", model), ("warmup_steps", warmup_steps), ("dtype", dtype),
+                            ("device", device), ("profiler", profiler), ("group", group),
+                            ("num_shards", num_shards), ("dp_ind", shard_id),
+                            ("opt_disable_delayed_grad_clipping", opt_disable_delayed_grad_clipping),
+                            ("opt_use_two_step_grad_clipping", opt_use_two_step_grad_clipping),
+                            ("opt_use_chunked_allreduce", opt_use_chunked_allreduce),
+                            ("tensor_parallelism", tensor_parallelism), ("tp_ind", tp_ind),
+                            ("tp_group", tp_group), ("expert_parallelism", expert_parallelism),
+                            ("ep_ind", ep_ind), ("ep_group", ep_group), ("dpep_ind", dpep_ind),
+                            ("dpep_group", dpep_group), ("skip_optimizer_step", skip_optimizer_step)):
+            setattr(self, name, value)
+        self.step_id = 0
         self.opt_store_clipped_grads = True   # leave flat_grad clipped after step(), as the reference does
-        owned = {id(p) for p in self.param_list}
-        model_params = list(self.model.parameters()) if self.model is not None else self.param_list
-        if self.flat_param_size > 0 and len(model_params) == len(owned) \
-                and all(id(p) in owned for p in model_params):
-            self._norm_plan = GradNormPlan(self.param_start_inds, self.param_sizes, self.device)
+
+        # layout: one running offset over the group's parameters
+        self.param_list = list(self.param_groups[0]["params"])
+        self.param_sizes, self.param_start_inds, offset = [], [], 0
+        for p in self.param_list:
+            self.param_start_inds.append(offset)
+            self.param_sizes.append(p.numel())
+            offset += p.numel()
+        self.flat_param_size = offset
+
+        def buffer(dt, zero=True):
+            make = torch.zeros if zero else torch.empty
+            return make(self.flat_param_size, dtype=dt, device=device)
+
+        keep_state = not skip_optimizer_step
+        self.flat_param = buffer(dtype, zero=False)
+        self.flat_grad = buffer(dtype)
+        self.flat_exp_avg = buffer(torch.float32) if keep_state else None
+        self.flat_exp_avg_sq = buffer(torch.float32) if keep_state else None
+
+        # move the parameters in: their values first, then re-point data and grad at the slices
+        if self.param_list:
+            slices = self.flat_param.split(self.param_sizes)
+            grad_slices = self.flat_grad.split(self.param_sizes)
+            with torch.no_grad():
+                for p, dst, gdst in zip(self.param_list, slices, grad_slices):
+                    dst = dst.view(p.shape)
+                    dst.copy_(p.data)
+                    p.data = dst
+                    p.grad = gdst.view(p.shape)
+        if dtype == torch.float32:
+            self.flat_fp32_master_param = self.flat_param          # one buffer serves as both
+        elif keep_state:
+            self.flat_fp32_master_param = self.flat_param.to(torch.float32)   # exact widening, one pass
         else:
-            self._norm_plan = None
+            self.flat_fp32_master_param = None
+
+        self._norm_plan = GradNormPlan(self.param_start_inds, self.param_sizes, device) \
+            if self.flat_param_size > 0 else None
+        self._foreign_plans = {}
 
     def zero_grad(self):
         self.flat_grad.zero_()
 
+    def _foreign_grads(self):
+        """Gradients of model parameters that this optimizer does not hold in flat_grad (the
+        reference takes the norm, and clips, over model.parameters(), optimizers.py:143-158)."""
+        if self.model is None:
+            return []
+        owned = {id(p) for p in self.param_list}
+        return [p.grad for p in self.model.parameters() if id(p) not in owned and p.grad is not None]
+
     def _grad_norm_and_clip(self):
         """Gradient norm (always) and the clip to 1.0 (after warm-up), reference
-        optimizers.py:136-160.  Returns (grad_norm, clip_coef): grad_norm is a 0-dim tensor in the
-        gradient dtype like torch.nn.utils.get_total_norm gives; clip_coef is a device fp32 scalar
-        for the update kernel to apply, or None when this step does not clip.  The single-step
-        and two-step variants of the reference compute the same thing on one device."""
+        optimizers.py:136-160.  Returns (grad_norm, clip_coef): grad_norm is a fresh 0-dim tensor in
+        the gradient dtype like torch.nn.utils.get_total_norm gives; clip_coef is a device fp32
+        scalar for the update kernel to apply, or None when this step does not clip.  The
+        single-step and two-step variants of the reference compute the same thing on one device.
+        Gradients outside flat_grad are measured by the same kernels (one extra launch per tensor)
+        and scaled in place here, since no update kernel touches them."""
         clip_now = self.opt_disable_delayed_grad_clipping or (self.step_id >= self.warmup_steps)
-        if self._norm_plan is None:
-            # the model holds parameters this optimizer does not own: their gradients are not in
-            # flat_grad, so take the norm over the model's list with the library calls
-            grads = [p.grad for p in self.model.parameters() if p.grad is not None]
-            grad_norm = torch.nn.utils.get_total_norm(grads)
-            if clip_now:
-                torch.nn.utils.clip_grads_with_norm_(self.model.parameters(), 1.0, grad_norm)
-            return grad_norm, None
-        total, coef = self._norm_plan.run(self.flat_grad, max_norm=1.0)
-        return total.to(self.flat_grad.dtype), (coef if clip_now else None)
+        foreign = self._foreign_grads()
+        if self._norm_plan is None and not foreign:
+            zero = torch.zeros((), dtype=self.flat_grad.dtype, device=self.device)
+            return zero, None
+        total, coef = run_grad_norm(self._norm_plan, self.flat_grad, foreign, self._foreign_plans,
+                                    max_norm=1.0)
+        if clip_now:
+            for g in foreign:
+                scale_grad_(g, coef)
+        return total.to(self.flat_grad.dtype, copy=True), (coef if clip_now else None)
 
     def step(self, closure=None):
         with record_pcl_function("4opt-step_grad-clip"):
             grad_norm, clip_coef = self._grad_norm_and_clip()
 
         with record_pcl_function("4opt-step_compute"):
-            if not self.skip_optimizer_step:
+            if self.flat_param_size == 0:
+                pass
+            elif not self.skip_optimizer_step:
+                group = self.param_groups[0]
                 beta1, beta2 = self.defaults["betas"]
-                eps = self.defaults["eps"]
-                lr = self.param_groups[0]["lr"]
-                weight_decay = self.defaults["weight_decay"]
                 adamw_step_(self.flat_param, self.flat_grad, self.flat_fp32_master_param,
-                            self.flat_exp_avg, self.flat_exp_avg_sq, self.step_id + 1, lr, beta1,
-                            beta2, eps, weight_decay, grad_scale=clip_coef,
-                            store_scaled_grad=self.opt_store_clipped_grads)
+                            self.flat_exp_avg, self.flat_exp_avg_sq, self.step_id + 1, group["lr"], beta1,
+                            beta2, self.defaults["eps"], self.defaults["weight_decay"],
+                            grad_scale=clip_coef, store_scaled_grad=self.opt_store_clipped_grads)
             elif clip_coef is not None:
-                # no update kernel to fold the clip into
-                self.flat_grad.mul_(clip_coef.to(self.flat_grad.dtype))
-        # Update step
+                scale_grad_(self.flat_grad, clip_coef)   # no update kernel to fold the clip into
         self.step_id += 1
-
         return grad_norm
 
     def state_dict(self):
-        opt_state_dict = {
-            "flat_exp_avg": self.flat_exp_avg,
-            "flat_exp_avg_sq": self.flat_exp_avg_sq,
-            "flat_fp32_master_param": self.flat_fp32_master_param,
-            "step_id": self.step_id
-        }
-        return opt_state_dict
+        state = {key: getattr(self, key) for key in _STATE_KEYS}
+        state["step_id"] = self.step_id
+        return state
 
     def load_state_dict(self, opt_state_dict):
-        self.flat_exp_avg.copy_(opt_state_dict["flat_exp_avg"].to(self.device))
-        self.flat_exp_avg_sq.copy_(opt_state_dict["flat_exp_avg_sq"].to(self.device))
-        self.flat_fp32_master_param.copy_(opt_state_dict["flat_fp32_master_param"].to(self.device))
+        for key in _STATE_KEYS:
+            getattr(self, key).copy_(opt_state_dict[key].to(self.device))
         self.step_id = opt_state_dict["step_id"]
 
 
@@ -262,6 +249,71 @@ class GradNormPlan:
         lib = _n.lib()
         _n.check(lib.om_grad_sumsq(_n.ptr(flat_grad), code, _n.ptr(self.chunk_offsets), self.n_chunks,
                                    _n.ptr(self.partials), _n.stream()), "om_grad_sumsq")
+        _n.check(lib.om_grad_norm_clip_coef(_n.ptr(self.partials), _n.ptr(self.seg_first_chunk),
+                                            self.n_segs, code, float(max_norm), _n.ptr(self.seg_norms),
+                                            _n.ptr(self.out), _n.ptr(self.out) + 4, _n.stream()),
+                 "om_grad_norm_clip_coef")
+        return self.out[0], self.out[1:2]
+
+
+def scale_grad_(grad, coef):
+    """grad = cast(grad * coef) in place, coef a device fp32 scalar: the multiply of
+    clip_grads_with_norm_ (reference optimizers.py:145/150/154) for a tensor no update kernel reads."""
+    _n.require_cuda_contiguous(grad, coef)
+    if coef.dtype != torch.float32 or coef.numel() != 1:
+        raise TypeError("coef must be one float32 element on the device")
+    _n.check(_n.lib().om_grad_scale(_n.ptr(grad), grad.numel(), _n.dtype_code(grad), _n.ptr(coef),
+                                    _n.stream()), "om_grad_scale")
+
+
+def run_grad_norm(plan, flat_grad, foreign, cache, max_norm=1.0):
+    """Total gradient norm and clip coefficient over flat_grad's parameters (through `plan`, may be
+    None) followed by the tensors in `foreign`, each counted as one more parameter.  `cache` keeps
+    the foreign tensors' chunk tables between steps."""
+    if not foreign:
+        return plan.run(flat_grad, max_norm)
+    dtype = flat_grad.dtype
+    for g in foreign:
+        if g.dtype != dtype:
+            raise TypeError("all gradients must share the optimizer's dtype")
+    key = tuple((g.data_ptr(), g.numel()) for g in foreign)
+    joint = cache.get(key)
+    if joint is None:
+        cache.clear()
+        joint = cache[key] = JointGradNormPlan(plan, [g.numel() for g in foreign], flat_grad.device)
+    return joint.run(flat_grad, foreign, max_norm)
+
+
+class JointGradNormPlan:
+    """One partial-sum table over flat_grad's chunks followed by the chunks of some separate
+    gradient tensors; a single om_grad_norm_clip_coef over all of them."""
+
+    def __init__(self, plan, foreign_sizes, device):
+        self.flat = plan
+        base_chunks = plan.n_chunks if plan is not None else 0
+        first = plan.seg_first_chunk.cpu().tolist() if plan is not None else [0]
+        self.tensors = []
+        for size in foreign_sizes:
+            sub = GradNormPlan([0], [size], device)
+            self.tensors.append((sub, first[-1]))
+            first.append(first[-1] + sub.n_chunks)
+        self.n_chunks, self.n_segs = first[-1], len(first) - 1
+        assert self.n_chunks >= base_chunks
+        self.seg_first_chunk = torch.tensor(first, dtype=torch.int64).to(device)
+        self.partials = torch.empty(max(self.n_chunks, 1), dtype=torch.float32, device=device)
+        self.seg_norms = torch.empty(self.n_segs, dtype=torch.float32, device=device)
+        self.out = torch.empty(2, dtype=torch.float32, device=device)
+
+    def run(self, flat_grad, foreign, max_norm=1.0):
+        lib = _n.lib()
+        code = _n.dtype_code(flat_grad)
+        if self.flat is not None:
+            _n.check(lib.om_grad_sumsq(_n.ptr(flat_grad), code, _n.ptr(self.flat.chunk_offsets),
+                                       self.flat.n_chunks, _n.ptr(self.partials), _n.stream()), "om_grad_sumsq")
+        for g, (sub, at) in zip(foreign, self.tensors):
+            _n.require_cuda_contiguous(g)
+            _n.check(lib.om_grad_sumsq(_n.ptr(g), code, _n.ptr(sub.chunk_offsets), sub.n_chunks,
+                                       _n.ptr(self.partials) + 4 * at, _n.stream()), "om_grad_sumsq")
         _n.check(lib.om_grad_norm_clip_coef(_n.ptr(self.partials), _n.ptr(self.seg_first_chunk),
                                             self.n_segs, code, float(max_norm), _n.ptr(self.seg_norms),
                                             _n.ptr(self.out), _n.ptr(self.out) + 4, _n.stream()),

@@ -147,7 +147,8 @@ from oracle import moe_layer as L      # noqa: E402
 from oracle import routing as R        # noqa: E402
 from util import assert_bf16_parity    # noqa: E402
 
-SAMPLE_BARS = {"out": (6.0, 1e-2), "grad": (6.0, 1e-2), "wgrad": (6.0, 1e-2)}
+# measured: out 1.95-2.29 x the bf16 floor, dx 2.8-3.2 x, d routing weights 2.5 x, expert dW 1.4-2.7 x
+SAMPLE_BARS = {"out": (2.6, 3.5e-3), "grad": (3.5, 5e-3), "wgrad": (3.2, 4.5e-3)}
 
 
 def _expert_wgrads(x, dout, tok, w_tok, wg, wu, wd):

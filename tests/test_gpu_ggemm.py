@@ -12,8 +12,10 @@ import torch
 
 from util import assert_bf16_parity, max_abs, mean_rel
 
-ONE_ROUNDING = (1.1, 2.5e-3)          # (excess over the bf16 floor, absolute cap on mean_rel)
-MLP_BARS = {"out": (6.0, 1e-2), "grad": (6.0, 1e-2)}
+# (excess over the bf16 floor, absolute cap on mean_rel); measured: single products 1.00 x the floor,
+# the merged MLP 1.6 x (y) and 1.5-2.5 x (gradients)
+ONE_ROUNDING = (1.03, 1.8e-3)
+MLP_BARS = {"out": (1.9, 2.7e-3), "grad": (2.9, 4.1e-3)}
 
 pytestmark = pytest.mark.gpu
 

@@ -163,3 +163,55 @@ def test_optimizer_step_clips_like_the_reference_sequence(cuda, oracle_lib, warm
     # the model's parameters are still views of the flat buffer
     first = next(iter(net.parameters()))
     assert first.data_ptr() == opt.flat_param.data_ptr()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_returned_norm_is_not_overwritten_by_the_next_step(cuda, dtype):
+    """step() hands back a tensor of its own (the reference returns get_total_norm's fresh result,
+    optimizers.py:136-158): a training loop that keeps the norms of several steps must not see the
+    first one change when the second step runs."""
+    from optimus.optimizers import MixedPrecisionAdamW
+    torch.manual_seed(5)
+    net = _Net().to(dtype).to(cuda)
+    opt = MixedPrecisionAdamW(net.parameters(), net, lr=1e-3, dtype=dtype, device=cuda, warmup_steps=10**9)
+    opt.flat_grad.copy_(_grad(opt.flat_param_size, dtype, 1, 1.0))
+    first = opt.step()
+    kept = float(first)
+    opt.flat_grad.copy_(_grad(opt.flat_param_size, dtype, 2, 3.0))
+    second = opt.step()
+    torch.cuda.synchronize()
+    assert float(first) == kept and abs(float(second) - 3.0 * kept) < 0.1 * kept
+    assert first.data_ptr() != second.data_ptr() and first.dtype == dtype
+
+
+@pytest.mark.parametrize("clip", [True, False])
+def test_parameters_outside_the_optimizer_count_in_norm_and_clip(cuda, clip):
+    """A model with parameters the optimizer was not given: the reference takes the norm and clips
+    over model.parameters() (optimizers.py:143-158), so their gradients count and are scaled too.
+    Checked against the same library calls on CPU copies."""
+    from optimus.optimizers import MixedPrecisionAdamW
+    torch.manual_seed(3)
+    net = _Net().to(torch.bfloat16).to(cuda)
+    owned = [net.a.weight, net.a.bias]
+    opt = MixedPrecisionAdamW(owned, net, lr=1e-3, dtype=torch.bfloat16, device=cuda,
+                              warmup_steps=0 if clip else 10**9)
+    g = torch.Generator().manual_seed(8)
+    for p in net.parameters():
+        val = torch.randn(p.shape, generator=g).to(torch.bfloat16).to(cuda)
+        if p.grad is None:
+            p.grad = val
+        else:
+            p.grad.copy_(val)
+    cpu = [p.grad.detach().cpu().clone() for p in net.parameters()]
+    want = torch.nn.utils.get_total_norm(cpu)
+    if clip:
+        holders = [torch.nn.Parameter(torch.empty_like(t)) for t in cpu]
+        for h, t in zip(holders, cpu):
+            h.grad = t
+        torch.nn.utils.clip_grads_with_norm_(holders, 1.0, want)
+    norm = opt.step()
+    torch.cuda.synchronize()
+    assert float(norm) == float(want)
+    for p, t in zip(net.parameters(), cpu):
+        assert torch.equal(p.grad.cpu(), t), "gradient after step() differs from the library sequence"
+    assert float(want) > 1.0

@@ -21,9 +21,11 @@ pytestmark = pytest.mark.gpu
 
 MAX_ABS = 2e-2
 # (excess over the bf16 floor, absolute cap on mean_rel) for the layer's output and its gradients
-LAYER_BARS = {"out": (6.0, 1e-2), "grad": (6.0, 1e-2)}
-ODD_BARS = {"out": (6.0, 1e-2), "grad": (8.0, 1.5e-2)}
-DSV3_GATE_BAR = (12.0, 2e-2)
+# Measured on MI355X: out 1.8-2.3 x the floor (2.5-3.2e-3), gradients 1.5-3.2 x (2.2-4.5e-3).
+LAYER_BARS = {"out": (2.6, 3.5e-3), "grad": (3.5, 5e-3)}
+# tiny token counts: the gate weight's gradient is a sum of as few as three rounded terms (6.3 x)
+ODD_BARS = {"out": (2.6, 3.5e-3), "grad": (4.0, 5.5e-3), "gate_w": (7.0, 1e-2)}
+DSV3_GATE_BAR = (3.5, 5e-3)
 
 
 def _olmoe_block(inp, cuda, fast=True, merged=True, fp32_logits=True):
@@ -126,7 +128,7 @@ def test_fast_block_odd_small_shapes(cuda, T, H, I, N, K, renorm):
            "w_gate": blk.experts.gate_proj_merged_weight.grad, "w_up": blk.experts.up_proj_merged_weight.grad,
            "w_down": blk.experts.down_proj_merged_weight.grad}
     for k, gref in ref_grads.items():
-        assert_bf16_parity(got[k], gref, *ODD_BARS["grad"], tag=f"{tag} d{k}",
+        assert_bf16_parity(got[k], gref, *ODD_BARS["gate_w" if k == "gate_w" else "grad"], tag=f"{tag} d{k}",
                            max_abs_bar=MAX_ABS * max(1.0, float(gref.abs().max())))
 
 

@@ -81,7 +81,8 @@ def _reference(c, residual=False):
     return [out.detach()] + grads
 
 
-ROUTED_BARS = {"out": (6.0, 1e-2), "grad": (8.0, 1.5e-2)}
+# (excess over one ideal bf16 rounding, cap); measured: out 1.0-2.0 x, gradients 1.55-2.7 x
+ROUTED_BARS = {"out": (2.3, 3.2e-3), "grad": (3.1, 4.4e-3)}
 NAMES = ("out", "dx", "d_routing_weights", "dw_gate", "dw_up", "dw_down", "d_residual")
 
 
