@@ -218,6 +218,22 @@ int om_moe_sort(const void *selected_experts, int index_dtype, int64_t T, int K,
                 int32_t *selected_experts_indices, void *workspace, int64_t workspace_bytes,
                 void *stream);
 
+/* om_moe_sort_static: om_moe_sort without a workspace argument and without any allocation.  It has
+ * no counterpart in the reference; it is for callers that cannot allocate device memory or carry a
+ * workspace around: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  The block table that om_moe_sort keeps in the caller's workspace lives in a fixed
+ * array of om_moe_sort_static_capacity_bytes() (4 MiB) inside the library, one copy per GPU, held
+ * until the process ends.  Inputs whose om_moe_sort_workspace_bytes(T, K, NR) exceeds that capacity
+ * return OM_ERR_WORKSPACE (4 MiB serves e.g. 8M pairs over 256 local experts).  Same results as
+ * om_moe_sort, bit for bit.  The array is shared by every call on a GPU: calls that overlap on one
+ * GPU (two streams, two threads) race; calls on one stream are ordered and safe.  Nothing in the
+ * array needs to start at zero.                                                             */
+int64_t om_moe_sort_static_capacity_bytes(void);
+int om_moe_sort_static(const void *selected_experts, int index_dtype, int64_t T, int K,
+                       int expert_start_idx, int expert_end_idx, int32_t *cum_token_counts,
+                       int32_t *cum_expert_counts_ep, int32_t *input_indices, int32_t *output_indices,
+                       int32_t *selected_experts_indices, void *stream);
+
 /* The reference's two index kernels with their own table layout, for callers of the
  * pybind module that still run K2 (torch.cumsum) themselves.
  * replaces: compute_partial_token_counts      sparse_moe_block.sycl:138-173

@@ -10,6 +10,7 @@
 // deterministic.
 // Also: the reference's two index kernels with their own [expert][column] table layout.
 #include "common.h"
+#include <mutex>
 
 namespace {
 
@@ -263,25 +264,19 @@ extern "C" int64_t om_moe_sort_workspace_bytes(int64_t T, int K, int NR) {
     return (NB * NR + NB + 1) * static_cast<int64_t>(sizeof(int32_t));
 }
 
-extern "C" int om_moe_sort(const void *selected_experts, int index_dtype, int64_t T, int K,
-                           int expert_start_idx, int expert_end_idx, int32_t *cum_token_counts,
-                           int32_t *cum_expert_counts_ep, int32_t *input_indices,
-                           int32_t *output_indices, int32_t *selected_experts_indices,
-                           void *workspace, int64_t workspace_bytes, void *stream) {
-    if (index_dtype != OM_I32 && index_dtype != OM_I64) return OM_ERR_DTYPE;
+namespace {
+
+// Launches count, scan and scatter with `workspace` holding the [NB][NR] block table and the
+// [NB] kept-pair bases.  Arguments are validated by the two entry points below.
+int moe_sort_launch(const void *selected_experts, int index_dtype, int64_t T, int K,
+                    int expert_start_idx, int expert_end_idx, int32_t *cum_token_counts,
+                    int32_t *cum_expert_counts_ep, int32_t *input_indices, int32_t *output_indices,
+                    int32_t *selected_experts_indices, int32_t *workspace, hipStream_t st) {
     const int NR = expert_end_idx - expert_start_idx;
-    if (T < 0 || K < 1 || NR < 1 || NR > SORT_MAX_NR || expert_start_idx < 0) return OM_ERR_SHAPE;
     const int64_t n_pairs = T * K;
-    if (n_pairs > 0x7fffffffLL) return OM_ERR_SHAPE;
-    if (!cum_token_counts || !cum_expert_counts_ep) return OM_ERR_NULL;
-    if (T > 0 && (!selected_experts || !input_indices || !output_indices || !selected_experts_indices))
-        return OM_ERR_NULL;
     const int64_t NB = (n_pairs + SORT_CHUNK - 1) / SORT_CHUNK;
-    if (workspace_bytes < om_moe_sort_workspace_bytes(T, K, NR)) return OM_ERR_WORKSPACE;
-    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 3u)) return OM_ERR_ALIGN;
-    int32_t *block_hist = static_cast<int32_t *>(workspace);
+    int32_t *block_hist = workspace;
     int32_t *hits_base = block_hist + NB * NR;
-    hipStream_t st = om_stream(stream);
     const int nbits = key_bits(NR);
     const size_t lds_count = static_cast<size_t>(SORT_WAVES) * NR * sizeof(int);
     const size_t lds_scatter = lds_count + SORT_WAVES * sizeof(int);
@@ -310,6 +305,93 @@ extern "C" int om_moe_sort(const void *selected_experts, int index_dtype, int64_
                 output_indices, selected_experts_indices);
     }
     return om_launch_status();
+}
+
+int moe_sort_check(const void *selected_experts, int index_dtype, int64_t T, int K,
+                   int expert_start_idx, int expert_end_idx, const int32_t *cum_token_counts,
+                   const int32_t *cum_expert_counts_ep, const int32_t *input_indices,
+                   const int32_t *output_indices, const int32_t *selected_experts_indices) {
+    if (index_dtype != OM_I32 && index_dtype != OM_I64) return OM_ERR_DTYPE;
+    const int NR = expert_end_idx - expert_start_idx;
+    if (T < 0 || K < 1 || NR < 1 || NR > SORT_MAX_NR || expert_start_idx < 0) return OM_ERR_SHAPE;
+    if (T * K > 0x7fffffffLL) return OM_ERR_SHAPE;
+    if (!cum_token_counts || !cum_expert_counts_ep) return OM_ERR_NULL;
+    if (T > 0 && (!selected_experts || !input_indices || !output_indices || !selected_experts_indices))
+        return OM_ERR_NULL;
+    return OM_OK;
+}
+
+}  // namespace
+
+extern "C" int om_moe_sort(const void *selected_experts, int index_dtype, int64_t T, int K,
+                           int expert_start_idx, int expert_end_idx, int32_t *cum_token_counts,
+                           int32_t *cum_expert_counts_ep, int32_t *input_indices,
+                           int32_t *output_indices, int32_t *selected_experts_indices,
+                           void *workspace, int64_t workspace_bytes, void *stream) {
+    const int rc = moe_sort_check(selected_experts, index_dtype, T, K, expert_start_idx, expert_end_idx,
+                                  cum_token_counts, cum_expert_counts_ep, input_indices, output_indices,
+                                  selected_experts_indices);
+    if (rc != OM_OK) return rc;
+    if (workspace_bytes < om_moe_sort_workspace_bytes(T, K, expert_end_idx - expert_start_idx))
+        return OM_ERR_WORKSPACE;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 3u)) return OM_ERR_ALIGN;
+    return moe_sort_launch(selected_experts, index_dtype, T, K, expert_start_idx, expert_end_idx,
+                           cum_token_counts, cum_expert_counts_ep, input_indices, output_indices,
+                           selected_experts_indices, static_cast<int32_t *>(workspace), om_stream(stream));
+}
+
+// ---- om_moe_sort for callers that cannot allocate ----------------------------------------------
+// The block table lives in a file-scope device array instead of a caller's workspace.  The array's
+// name is only a host-side handle: its device address is asked from the runtime once per device
+// (with that device current) and kept; kernels and everything else in host code use that address.
+constexpr int64_t SORT_SCRATCH_BYTES = 4ll << 20;
+constexpr int SORT_MAX_DEVICES = 64;
+
+static __device__ __align__(256) int32_t sort_scratch[SORT_SCRATCH_BYTES / sizeof(int32_t)];
+
+namespace {
+
+std::mutex sort_scratch_mutex;
+int32_t *sort_scratch_ptr[SORT_MAX_DEVICES] = {};
+
+// Device address of sort_scratch on the current device; nullptr if the runtime refuses.
+int32_t *sort_scratch_on_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SORT_MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> lock(sort_scratch_mutex);
+    if (!sort_scratch_ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(sort_scratch)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        sort_scratch_ptr[dev] = static_cast<int32_t *>(p);
+    }
+    return sort_scratch_ptr[dev];
+}
+
+}  // namespace
+
+extern "C" int64_t om_moe_sort_static_capacity_bytes(void) { return SORT_SCRATCH_BYTES; }
+
+extern "C" int om_moe_sort_static(const void *selected_experts, int index_dtype, int64_t T, int K,
+                                  int expert_start_idx, int expert_end_idx, int32_t *cum_token_counts,
+                                  int32_t *cum_expert_counts_ep, int32_t *input_indices,
+                                  int32_t *output_indices, int32_t *selected_experts_indices,
+                                  void *stream) {
+    const int rc = moe_sort_check(selected_experts, index_dtype, T, K, expert_start_idx, expert_end_idx,
+                                  cum_token_counts, cum_expert_counts_ep, input_indices, output_indices,
+                                  selected_experts_indices);
+    if (rc != OM_OK) return rc;
+    if (om_moe_sort_workspace_bytes(T, K, expert_end_idx - expert_start_idx) > SORT_SCRATCH_BYTES)
+        return OM_ERR_WORKSPACE;
+    int32_t *scratch = sort_scratch_on_current_device();
+    if (!scratch) return OM_ERR_LAUNCH;
+    // count writes every cell of the block table it later reads and scan writes every base, so
+    // nothing left in the array by an earlier call needs clearing
+    return moe_sort_launch(selected_experts, index_dtype, T, K, expert_start_idx, expert_end_idx,
+                           cum_token_counts, cum_expert_counts_ep, input_indices, output_indices,
+                           selected_experts_indices, scratch, om_stream(stream));
 }
 
 extern "C" int om_compute_partial_token_counts(const void *selected_experts, int index_dtype,

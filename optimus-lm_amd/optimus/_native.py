@@ -63,6 +63,9 @@ SIGNATURES = {
     "om_moe_sort_workspace_bytes": (c_i64, [c_i64, c_int, c_int]),
     "om_moe_sort": (c_int, [c_void_p, c_int, c_i64, c_int, c_int, c_int, c_void_p, c_void_p,
                             c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_void_p]),
+    "om_moe_sort_static_capacity_bytes": (c_i64, []),
+    "om_moe_sort_static": (c_int, [c_void_p, c_int, c_i64, c_int, c_int, c_int, c_void_p, c_void_p,
+                                   c_void_p, c_void_p, c_void_p, c_void_p]),
     "om_compute_partial_token_counts": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
                                                 c_i64, c_int, c_i64, c_void_p]),
     "om_compute_input_and_output_indices": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p,
@@ -130,6 +133,7 @@ _lib = None
 launch_log = None
 launch_filter = None   # optional set of entry-point names: only these are timed while launch_log is set
 _UNTIMED = {"om_version", "om_arch", "om_strerror", "om_moe_sort_workspace_bytes",
+            "om_moe_sort_static_capacity_bytes",
             "om_router_balance_workspace_bytes", "om_rmsnorm_bwd_workspace_bytes",
             "om_router_gate_wgrad_workspace_bytes", "om_router_gate_logits_split_workspace_bytes",
             "om_merged_mlp_row_dot_parts"}
