@@ -257,6 +257,12 @@ def bench_adamw(args, device):
             st["param"], st["grad"], st["master"], st["exp_avg"], st["exp_avg_sq"], hp["step_id"] + 1,
             hp["lr"], hp["betas"][0], hp["betas"][1], hp["eps"], hp["weight_decay"], grad_scale=one,
             store_scaled_grad=store), ("om_adamw_step_clipped",))
+    # What the update's access pattern reaches on this GPU with the arithmetic taken out: the same
+    # 64-thread blocks, the same 14 B read + 14 B written per parameter, the same cache hints.
+    t_probe = timed(lambda: _native.check(_native.lib().om_adamw_traffic_probe(
+        _native.ptr(st["param"]), _native.ptr(st["grad"]), _native.ptr(st["master"]), _native.ptr(st["exp_avg"]),
+        _native.ptr(st["exp_avg_sq"]), n, _native.stream()), "om_adamw_traffic_probe"), ("om_adamw_traffic_probe",))
+    probe_gbs = 28.0 * n / t_probe / 1e9
     grad_clip = {
         "grad_norm_ms": round(t_norm * 1e3, 3), "grad_norm_gb_per_s": round(2.0 * n / t_norm / 1e9, 1),
         "clipped_step_ms": round(t_clip[True] * 1e3, 3),
@@ -273,7 +279,13 @@ def bench_adamw(args, device):
                                    "param/grad + fp32 master/m/v, step 100"},
             "roofline": {"bound": "hbm", "kernel": "om_adamw_step", "achieved": round(gbs, 1),
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
-                         "traffic": MEASURED_TRAFFIC_BYTES["om_adamw_step"], "bytes_per_param": 28, "kernel_avg_ms": round(avg_s * 1e3, 3)},
+                         "traffic": MEASURED_TRAFFIC_BYTES["om_adamw_step"], "bytes_per_param": 28, "kernel_avg_ms": round(avg_s * 1e3, 3),
+                         "streaming_ceiling": {
+                             "what": "om_adamw_traffic_probe: the update kernel's loads and stores (14 B read + "
+                                     "14 B written per parameter, same block shape and cache hints) without "
+                                     "the arithmetic, same buffers, same process",
+                             "gb_per_s": round(probe_gbs, 1), "frac_of_peak": round(probe_gbs / PEAK_HBM_GBS, 4),
+                             "update_over_probe": round(gbs / probe_gbs, 4)}},
             "grad_clip": grad_clip}
 
 

@@ -63,6 +63,15 @@ int om_adamw_step(void *param, const void *grad, float *master, float *exp_avg,
                   double eps, double weight_decay, int64_t step, int param_dtype,
                   void *stream);
 
+/* om_adamw_traffic_probe: the loads and stores of om_adamw_step in bf16 mode (14 B read and 14 B
+ * written per element, same kernel shape and cache hints) with the arithmetic left out: master,
+ * exp_avg and exp_avg_sq are written back as read and param = bf16(master), which is what the
+ * optimizer keeps there anyway.  It has no counterpart in the reference; it exists so that a
+ * benchmark can state what this access pattern reaches on the GPU at hand next to the update
+ * itself.  n a multiple of 4 (a shorter tail is left untouched).                              */
+int om_adamw_traffic_probe(void *param, const void *grad, float *master, float *exp_avg,
+                           float *exp_avg_sq, int64_t n, void *stream);
+
 /* ------------------------------------------------------------------------------------
  * Gradient norm and clip coefficient over the flat gradient buffer
  * replaces: the "4opt-step_grad-clip" block of MixedPrecisionAdamW.step,

@@ -75,7 +75,7 @@ __global__ __launch_bounds__(256) void grad_sumsq_kernel(const T *__restrict__ g
         u32x4 q[4];
 #pragma unroll
         for (int u = 0; u < 4; u++)
-            if (j + u * 256 < nv) q[u] = vp[j + u * 256];
+            if (j + u * 256 < nv) q[u] = __builtin_nontemporal_load(vp + j + u * 256);   // read once
 #pragma unroll
         for (int u = 0; u < 4; u++)
             if (j + u * 256 < nv) {

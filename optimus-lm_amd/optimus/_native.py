@@ -27,6 +27,7 @@ SIGNATURES = {
     "om_strerror": (ctypes.c_char_p, [c_int]),
     "om_adamw_step": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_double,
                               c_double, c_double, c_double, c_double, c_i64, c_int, c_void_p]),
+    "om_adamw_traffic_probe": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_void_p]),
     "om_grad_sumsq": (c_int, [c_void_p, c_int, c_void_p, c_i64, c_void_p, c_void_p]),
     "om_grad_norm_clip_coef": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_double, c_void_p, c_void_p,
                                        c_void_p, c_void_p]),
