@@ -136,7 +136,7 @@ int om_route_softmax_topk_bwd(const void *logits, int logits_dtype, const int64_
  *   bf16 before the softmax) and written to logits_out [T,N] fp32 when it is not null (the
  *   backward and output_router_logits need them).  N <= 256, K <= min(N,64), H a multiple of 512
  *   (256 for N > 64, 64 for N > 128); other shapes return OM_ERR_SHAPE and the caller uses the
- *   two-step form (library GEMM + om_route_softmax_topk).
+ *   two-step form (om_router_gate_logits[_split] + om_route_softmax_topk).
  * om_router_gate_logits is the projection alone, for routers that score the fp32 logits
  *   differently (optimus/models/deepseek_v3/modeling_deepseek_v3.py:160 casts both operands to
  *   float32 and calls F.linear).                                                          */
@@ -162,14 +162,25 @@ int om_router_gate_logits_split(const void *x, const void *gate_weight, int64_t 
  * (optimus/models/common/moe.py:456, optimus/models/olmoe/modeling_olmoe.py:284) from the
  * gradient of the logits.  x [T,H] bf16; dlogits [T,N] fp32, rounded to bf16 as it is loaded;
  * products accumulate in fp32 over token ranges and the partial sums are added in a fixed order
- * (deterministic).  dweight [N,H] in dweight_dtype (OM_BF16 / OM_F32).  N in {32,64,128,256},
- * H a multiple of 128; other shapes return OM_ERR_SHAPE and the caller uses a library GEMM.
+ * (deterministic).  dweight [N,H] in dweight_dtype (OM_BF16 / OM_F32).  N <= 256, H a multiple
+ * of 128; other shapes return OM_ERR_SHAPE.
  * workspace: om_router_gate_wgrad_workspace_bytes(T,H,N) bytes of device memory, 16-byte
  * aligned (negative = error code).                                                        */
 int64_t om_router_gate_wgrad_workspace_bytes(int64_t T, int H, int N);
 int om_router_gate_wgrad(const void *x, const float *dlogits, int64_t T, int H, int N,
                          void *dweight, int dweight_dtype, void *workspace,
                          int64_t workspace_bytes, void *stream);
+
+/* om_router_gate_dgrad: gradient of the gate's input,
+ *   dx[t,h] = (base[t,h] +) sum_n bf16(dlogits[t,n]) * gate_weight[n,h]
+ * what autograd computes for the same nn.Linear (mm(dlogits, weight)), optionally with the
+ * accumulation into the tensor's other gradient folded in: `base` [T,H] bf16 (may be null, may be
+ * dx itself) is the gradient that reached hidden_states through the experts, and
+ * dx = bf16(float(base) + float(bf16(sum))) keeps both roundings of "matmul, then add".
+ * dlogits [T,N] fp32 (rounded to bf16 as it is loaded), gate_weight [N,H] bf16, dx [T,H] bf16.
+ * N <= 256, H a multiple of 8; other shapes return OM_ERR_SHAPE.                             */
+int om_router_gate_dgrad(const float *dlogits, const void *gate_weight, const void *base, void *dx,
+                         int64_t T, int H, int N, void *stream);
 
 /* Load-balancing statistics of one layer's router logits
  * replaces: the per-token part of load_balancing_loss_func,
@@ -248,7 +259,8 @@ int om_moe_sort_static(const void *selected_experts, int index_dtype, int64_t T,
  * replaces: compute_partial_token_counts      sparse_moe_block.sycl:138-173
  *           compute_input_and_output_indices  sparse_moe_block.sycl:217-280
  * partial_token_counts [NR,TH] and input_increment_buffer [NR,TH] are pre-zeroed by the
- * caller and updated in place; TB = T / TH tokens per table column (T % TH == 0).        */
+ * caller and updated in place; TB = T / TH tokens per table column (T % TH == 0, any TB; the
+ * reference fixes TB = 8).  One wavefront per column; NR <= 1024.                           */
 int om_compute_partial_token_counts(const void *selected_experts, int index_dtype,
                                     int32_t *partial_token_counts, int32_t *expert_counts_ep,
                                     int expert_start_idx, int expert_end_idx, int64_t T, int K,
@@ -341,8 +353,10 @@ int om_rmsnorm_bwd(const void *dy, const void *h, const void *weight, const floa
  *   om_grouped_gemm_wgrad  dW[g]       = dout[s:e,:].T @ in[s:e,:]  (zeros when s == e)
  * w_stride: elements between the matrices of consecutive experts in `weight` /
  * `weight_grad`; 0 means densely packed (N*K, the merged [G,N,K] layout).  A larger stride
- * serves per-expert nn.Linear weights that sit at a constant pitch inside one flat buffer.
- * N and K must be multiples of 128.  fwd and dgrad (and the merged-MLP fusions below) keep
+ * serves per-expert nn.Linear weights that sit at a constant pitch inside one flat buffer
+ * (a multiple of 8 elements, else OM_ERR_ALIGN).  N and K must be multiples of 128.  Every
+ * activation / weight tensor spans fewer than 2^35 elements (the kernels address operands in
+ * 32-bit units of 16 bytes), e.g. 16M routed rows of 2048.  fwd and dgrad (and the merged-MLP fusions below) keep
  * a per-expert tile table in LDS and take G <= 1024 (OM_ERR_SHAPE above that); wgrad has no
  * such limit.                                                                             */
 int om_grouped_gemm_fwd(const void *input, const void *weight, void *output,

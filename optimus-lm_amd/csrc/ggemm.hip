@@ -60,21 +60,8 @@ constexpr int BK = 64;  // contraction step, elements
 // kernel on one box: the weight gradients gain 4 % with their split and the others lose 1-2 % with
 // it; an even spread over the step, everything in one place, or cutting through the A loads are
 // all 2-7 % worse on the whole layer.
-#ifndef OM_LD_T
-#define OM_LD_T 4
-#define OM_LD_0 4
-#define OM_LD_1 0
-#define OM_LD_2 0
-#endif
-#ifndef OM_LDW_T
-#define OM_LDW_T 0
-#define OM_LDW_0 4
-#define OM_LDW_1 4
-#define OM_LDW_2 0
-#endif
-#ifndef OM_ROT_MODE
-#define OM_ROT_MODE 1
-#endif
+constexpr int LD_SHARE_T = 4, LD_SHARE_0 = 4, LD_SHARE_1 = 0, LD_SHARE_2 = 0;       // fwd / dgrad
+constexpr int LDW_SHARE_T = 0, LDW_SHARE_0 = 4, LDW_SHARE_1 = 4, LDW_SHARE_2 = 0;   // wgrad
 constexpr int NUM_XCD = 8;
 
 struct GemmParams {
@@ -238,14 +225,8 @@ __device__ __forceinline__ bool find_tile(const int *tile_end, const int *seg, i
 // the expert's rows of both operands, and with near-uniform routing whole experts per XCD (what
 // equal tile counts give) is the better cut.  Every wavefront computes the two boundaries it needs
 // by itself from cum_token_counts (two strided passes, no LDS, no barrier).
-#ifndef OM_WGRAD_EPI_STEPS
-#define OM_WGRAD_EPI_STEPS 3
-#endif
-constexpr int WGRAD_EPILOGUE_STEPS = OM_WGRAD_EPI_STEPS;   // a tile's stores take about as long as 3 steps
-#ifndef OM_WGRAD_BALANCE_MAX_EXPERTS
-#define OM_WGRAD_BALANCE_MAX_EXPERTS 4096
-#endif
-constexpr int WGRAD_BALANCE_MAX_EXPERTS = OM_WGRAD_BALANCE_MAX_EXPERTS;
+constexpr int WGRAD_EPILOGUE_STEPS = 3;   // a tile's stores take about as long as 3 steps
+constexpr int WGRAD_BALANCE_MAX_EXPERTS = 4096;
 __device__ __forceinline__ int wgrad_tile_units(int rows, int bk) {
     const int steps = (rows + bk - 1) / bk;
     return ((steps + 1) & ~1) + WGRAD_EPILOGUE_STEPS;   // the main loop takes its steps in pairs
@@ -345,7 +326,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // ---- per-lane source offsets of the direct loads (elements, without the c0 term) ------------
     // CONTIG : lane -> (row = group*8 + lane/8, chunk = (lane%8) ^ swz(row))
     // STRIDED: lane -> (crow = group*(64/CPR) + lane/CPR, chunk = (lane%CPR) ^ ((crow&3)<<2))
-    int a_off[A_LOADS], b_off[B_LOADS];  // the host checks that every operand spans < 2^31 elements
+    // in units of 16 bytes (8 elements): every row pitch, expert pitch, tile origin and contraction
+    // step is a multiple of 8 elements, and the host checks that every operand spans < 2^32 units
+    uint32_t a_off[A_LOADS], b_off[B_LOADS];
     int a_crow[A_LOADS];  // STRIDED A in wgrad: c-row of the lane's slot (for the zero fill)
     int b_crow[B_LOADS];
     bool b_up[B_LOADS];   // EPI_SWIGLU: this LDS row comes from the up matrix
@@ -364,7 +347,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         b_up[i] = (EPI == EPI_SWIGLU) ? (((grp * 8 + (lane >> 3)) >> 5) & 1) : false;
     }
 
-    const int lda32 = static_cast<int>(p.lda), ldb32 = static_cast<int>(p.ldb);
+    const uint32_t lda16 = static_cast<uint32_t>(p.lda >> 3), ldb16 = static_cast<uint32_t>(p.ldb >> 3);
     // GATHER_B: the B rows that contraction step `step` needs, looked up one step ahead of the
     // loads that use them (plain loads: they land before the next wait for the direct loads).
     auto index_of = [&](int step, int c0, int c) -> int {   // c0: the step's first row (block-uniform)
@@ -435,11 +418,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         steps_per_phase = (c_len + BK - 1) / BK;
         total_steps = steps_per_phase * p.phases;
         loop_steps = (total_steps + 1) & ~1;
-#if OM_ROT_MODE
-        rot = ((OM_ROT_MODE == 1 ? rot_a : (rot_a >> 1)) + rot_b) % (steps_per_phase > 0 ? steps_per_phase : 1);
-#else
-        rot = 0;
-#endif
+        rot = (rot_a + rot_b) % (steps_per_phase > 0 ? steps_per_phase : 1);
 #pragma unroll
         for (int i = 0; i < A_LOADS; i++) {
             const int grp = wave * A_LOADS + i;
@@ -449,11 +428,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                 int64_t m = static_cast<int64_t>(row_begin) + row;
                 if (m >= row_end) m = row_end - 1;  // rows past the segment: valid memory, result unused
                 if (GATHER == GATHER_A) m = p.row_index[m];
-                a_off[i] = static_cast<int>(m * p.lda + ch * 8);
+                a_off[i] = static_cast<uint32_t>(((m * p.lda) >> 3) + ch);
             } else {
                 constexpr int CPR = BM / 8;
                 const int ch = (lane_s % CPR) ^ ((a_crow[i] & 3) << 2);
-                a_off[i] = row_begin + ch * 8;  // + (c_begin + c) * lda per step
+                a_off[i] = static_cast<uint32_t>((row_begin >> 3) + ch);  // + (c_begin + c) * lda16 per step
             }
         }
 #pragma unroll
@@ -466,14 +445,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                     // LDS rows alternate 32 gate rows / 32 up rows; the up matrix is B[1]
                     const int blk = row >> 5;
                     const int64_t n = n0 + (blk >> 1) * 32 + (row & 31);
-                    b_off[i] = static_cast<int>(expert * p.strideB + n * p.ldb + ch * 8);
+                    b_off[i] = static_cast<uint32_t>(((expert * p.strideB + n * p.ldb) >> 3) + ch);
                 } else {
-                    b_off[i] = static_cast<int>(expert * p.strideB + static_cast<int64_t>(n0 + row) * p.ldb + ch * 8);
+                    b_off[i] = static_cast<uint32_t>(((expert * p.strideB + static_cast<int64_t>(n0 + row) * p.ldb) >> 3) + ch);
                 }
             } else {
                 constexpr int CPR = BN / 8;
                 const int ch = (lane_s % CPR) ^ ((b_crow[i] & 3) << 2);
-                b_off[i] = static_cast<int>((EPI == EPI_WGRAD ? 0 : expert * p.strideB) + n0 + ch * 8);
+                b_off[i] = static_cast<uint32_t>((((EPI == EPI_WGRAD ? 0 : expert * p.strideB) + n0) >> 3) + ch);
             }
         }
         if (GATHER_W && expert != cached_expert) {
@@ -508,18 +487,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 #pragma unroll
         for (int i = 0; i < A_LOADS; i++) {
             if (i < lo || i >= hi) continue;
-            uint32_t off;  // bytes from the operand base; < 2^32 (checked on the host)
+            uint32_t off;  // 16-byte units from the operand base; < 2^32 (checked on the host)
             if (AKIND == CONTIG) {
-                off = static_cast<uint32_t>(a_off[i] + c0) * 2u;
+                off = a_off[i] + static_cast<uint32_t>(c0 >> 3);
             } else {
                 int c = c0 + a_crow[i];
                 if (EPI == EPI_WGRAD) c = min(c, c_len - 1);  // stay in the segment; zeroed below
                 if (GATHER == GATHER_WA)
-                    off = static_cast<uint32_t>(a_off[i] + a_src[GATHER == GATHER_WA ? i : 0] * lda32) * 2u;
+                    off = a_off[i] + static_cast<uint32_t>(a_src[GATHER == GATHER_WA ? i : 0]) * lda16;
                 else
-                    off = static_cast<uint32_t>(a_off[i] + (c_begin + c) * lda32) * 2u;
+                    off = a_off[i] + static_cast<uint32_t>(c_begin + c) * lda16;
             }
-            load16_to_lds(Ap + off, sa + i * 1024);
+            load16_to_lds(Ap + (static_cast<uint64_t>(off) << 4), sa + i * 1024);
         }
         if (hi >= A_LOADS && lo < A_LOADS) load_a_src(step + 1);   // this step's A loads are out
 #pragma unroll
@@ -527,16 +506,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             if (A_LOADS + i < lo || A_LOADS + i >= hi) continue;
             uint32_t off;
             if (BKIND == CONTIG) {
-                off = static_cast<uint32_t>(b_off[i] + c0) * 2u;
+                off = b_off[i] + static_cast<uint32_t>(c0 >> 3);
             } else {
                 int c = c0 + b_crow[i];
                 if (EPI == EPI_WGRAD) c = min(c, c_len - 1);
                 if (GATHER == GATHER_B)
-                    off = static_cast<uint32_t>(b_off[i] + b_src[GATHER == GATHER_B ? i : 0] * ldb32) * 2u;
+                    off = b_off[i] + static_cast<uint32_t>(b_src[GATHER == GATHER_B ? i : 0]) * ldb16;
                 else
-                    off = static_cast<uint32_t>(b_off[i] + (c_begin + c) * ldb32) * 2u;
+                    off = b_off[i] + static_cast<uint32_t>(c_begin + c) * ldb16;
             }
-            load16_to_lds(((EPI == EPI_SWIGLU && b_up[i]) ? Bup : Bp) + off, sb + i * 1024);
+            load16_to_lds(((EPI == EPI_SWIGLU && b_up[i]) ? Bup : Bp) + (static_cast<uint64_t>(off) << 4), sb + i * 1024);
         }
         if (hi >= A_LOADS + B_LOADS && lo < A_LOADS + B_LOADS) load_b_src(step + 1);   // this step's B loads are out
     };
@@ -547,11 +526,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // cycles, and a wavefront that has to wait for it cannot issue its MFMAs meanwhile.  Shares of
     // the NL loads: after the barrier of step s (stage free), then with slices 0, 1, 2 of step s+1.
     constexpr bool WG = EPI == EPI_WGRAD;
-    constexpr int LD_T = NL * (WG ? OM_LDW_T : OM_LD_T) / 8, LD_0 = NL * (WG ? OM_LDW_0 : OM_LD_0) / 8;
-    constexpr int LD_1 = NL * (WG ? OM_LDW_1 : OM_LD_1) / 8;
+    constexpr int LD_T = NL * (WG ? LDW_SHARE_T : LD_SHARE_T) / 8, LD_0 = NL * (WG ? LDW_SHARE_0 : LD_SHARE_0) / 8;
+    constexpr int LD_1 = NL * (WG ? LDW_SHARE_1 : LD_SHARE_1) / 8;
     constexpr int LD_2 = NL - LD_T - LD_0 - LD_1;
-    static_assert(OM_LD_T + OM_LD_0 + OM_LD_1 + OM_LD_2 == 8 && OM_LDW_T + OM_LDW_0 + OM_LDW_1 + OM_LDW_2 == 8 &&
-                      LD_2 >= 0, "load shares");
+    static_assert(LD_SHARE_T + LD_SHARE_0 + LD_SHARE_1 + LD_SHARE_2 == 8 &&
+                      LDW_SHARE_T + LDW_SHARE_0 + LDW_SHARE_1 + LDW_SHARE_2 == 8 && LD_2 >= 0, "load shares");
     // wgrad: zero the A c-rows past the end of the expert's rows (after the loads have landed,
     // before the barrier).  B holds finite in-segment data there, so the products vanish.
     auto zero_tail = [&](int step, char *stage) {
@@ -921,21 +900,30 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 // of 64x64) when an extent is not a multiple of 256 or experts hold few rows each.
 
 inline bool mult(int64_t v, int m) { return v > 0 && v % m == 0; }
-inline bool fits31(int64_t elems) { return elems >= 0 && elems < (1LL << 31); }
+// the kernels address an operand in 32-bit units of 16 bytes: fewer than 2^35 elements per tensor,
+// and per-expert pitches that are multiples of 8 elements (16-byte vectors need that anyway)
+inline bool fits_span(int64_t elems) { return elems >= 0 && elems < (1LL << 35); }
+inline bool pitch_ok(int64_t stride) { return stride >= 0 && stride % 8 == 0; }
 
-// wavefront grid of the 256x256 tile (overridable for tuning builds)
-#ifndef OM_WAVES_M
-#define OM_WAVES_M 2
-#endif
-#ifndef OM_WAVES_N
-#define OM_WAVES_N 4
-#endif
 // Blocks of a launch: one resident set (a multiple of the 8 XCDs), or fewer when there are few
 // tiles.  The 256x256 tile's 128 KB of LDS leave room for one block per CU, the 128x128 tile's
 // 64 KB for two.
-constexpr int NUM_CU = 256;
+// Compute units of the current device (256 on an MI355X in its default partition mode), asked from
+// the runtime once per device.
+inline int device_cu_count() {
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < NUM_XCD)
+            n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
 template <int BM> unsigned persistent_blocks(int64_t tiles) {
-    const int64_t per_xcd_max = (NUM_CU / NUM_XCD) * (BM == 256 ? 1 : 2);
+    const int64_t per_xcd_max = (device_cu_count() / NUM_XCD) * (BM == 256 ? 1 : 2);
     int64_t per_xcd = (tiles + NUM_XCD - 1) / NUM_XCD;
     if (per_xcd > per_xcd_max) per_xcd = per_xcd_max;
     if (per_xcd < 1) per_xcd = 1;
@@ -943,8 +931,8 @@ template <int BM> unsigned persistent_blocks(int64_t tiles) {
 }
 
 template <int BM> struct Waves {
-    static constexpr int M = (BM == 256) ? OM_WAVES_M : 2;
-    static constexpr int N = (BM == 256) ? OM_WAVES_N : 2;
+    static constexpr int M = 2;                       // 256x256: 2 x 4 wavefronts of 128x64;
+    static constexpr int N = (BM == 256) ? 4 : 2;    // 128x128: 2 x 2 wavefronts of 64x64
 };
 
 template <int BM, int BN, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = false>
@@ -991,7 +979,8 @@ extern "C" int om_grouped_gemm_fwd(const void *input, const void *weight, void *
     p.cum = cum_token_counts;
     p.lda = K; p.ldb = K; p.ldc = N;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(N) * K;
-    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
+    if (!pitch_ok(p.strideB)) return OM_ERR_ALIGN;
+    if (!fits_span(rows * K) || !fits_span(rows * N) || !fits_span(p.strideB * G)) return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = N; p.kc = K; p.phases = 1;
     return launch_rows_auto<CONTIG, CONTIG, EPI_STORE>(p, rows, om_stream(stream));
 }
@@ -1010,7 +999,8 @@ extern "C" int om_grouped_gemm_dgrad(const void *output_grad, const void *weight
     p.cum = cum_token_counts;
     p.lda = N; p.ldb = K; p.ldc = K;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(N) * K;
-    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
+    if (!pitch_ok(p.strideB)) return OM_ERR_ALIGN;
+    if (!fits_span(rows * K) || !fits_span(rows * N) || !fits_span(p.strideB * G)) return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
     return launch_rows_auto<CONTIG, STRIDED, EPI_STORE>(p, rows, om_stream(stream));
 }
@@ -1035,8 +1025,9 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inde
     p.row_index = index;
     p.lda = N; p.ldb = K; p.ldc = K;
     p.strideC = w_stride ? w_stride : static_cast<int64_t>(N) * K;
-    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideC * G) ||
-        !fits31(src_rows * (gather == GATHER_WA ? N : K)))
+    if (!pitch_ok(p.strideC)) return OM_ERR_ALIGN;
+    if (!fits_span(rows * K) || !fits_span(rows * N) || !fits_span(p.strideC * G) ||
+        !fits_span(src_rows * (gather == GATHER_WA ? N : K)))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
     hipStream_t st = om_stream(stream);
@@ -1116,7 +1107,8 @@ int gate_up_fwd_launch(const void *x, const int32_t *x_rows, int64_t src_rows, c
     p.row_scale = row_weights;
     p.lda = H; p.ldb = H; p.ldc = I;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(I) * H;
-    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G) || !fits31(src_rows * H))
+    if (!pitch_ok(p.strideB)) return OM_ERR_ALIGN;
+    if (!fits_span(rows * H) || !fits_span(rows * I) || !fits_span(p.strideB * G) || !fits_span(src_rows * H))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = I; p.kc = H; p.phases = 1;
     if (row_weights) return launch_rows_auto<CONTIG, CONTIG, EPI_SWIGLU, GATHER_A, true>(p, rows, om_stream(stream));
@@ -1186,7 +1178,8 @@ int down_dgrad_launch(const void *dy, const int32_t *dy_rows, int64_t src_rows, 
     p.row_dot = row_dot;
     p.lda = H; p.ldb = I; p.ldc = I;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(H) * I;
-    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G) || !fits31(src_rows * H))
+    if (!pitch_ok(p.strideB)) return OM_ERR_ALIGN;
+    if (!fits_span(rows * H) || !fits_span(rows * I) || !fits_span(p.strideB * G) || !fits_span(src_rows * H))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = I; p.kc = H; p.phases = 1;
     if (dy_rows) return launch_rows_auto<CONTIG, STRIDED, EPI_SWIGLU_BWD, GATHER_A, true>(p, rows, om_stream(stream));
@@ -1238,7 +1231,8 @@ extern "C" int om_merged_mlp_gate_up_dgrad(const void *dg, const void *du, const
     p.cum = cum_token_counts;
     p.lda = I; p.ldb = H; p.ldc = H;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(I) * H;
-    if (!fits31(rows * H) || !fits31(rows * I) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
+    if (!pitch_ok(p.strideB)) return OM_ERR_ALIGN;
+    if (!fits_span(rows * H) || !fits_span(rows * I) || !fits_span(p.strideB * G)) return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = H; p.kc = I; p.phases = 2;
     return launch_rows_auto<CONTIG, STRIDED, EPI_STORE>(p, rows, om_stream(stream));
 }

@@ -8,7 +8,8 @@
 // Ranks come from wavefront ballots (lanes holding the same expert form a mask; rank = popcount of
 // the mask below the lane), per-wave running offsets live in LDS: no atomics, so the result is
 // deterministic.
-// Also: the reference's two index kernels with their own [expert][column] table layout.
+// Also: the reference's two index operators with their own [expert][column] table layout, one
+// wavefront per column.
 #include "common.h"
 #include <mutex>
 
@@ -207,51 +208,104 @@ inline int key_bits(int NR) {  // keys 0..NR (NR = "not local")
     return b;
 }
 
-// ---- the reference's own index kernels (table layout [expert][column]) -----------------------
+// ---- the reference's table layout [expert][column] ---------------------------------------------
+// The pybind ops keep a table with one column per group of TB = T / TH consecutive tokens
+// (partial_token_counts [NR][TH], then its flattened cumsum, then a same-shaped table of running
+// increments).  Here one wavefront owns one column: its TB*K (token, k) pairs are walked in
+// row-major order 64 at a time, equal experts are matched by ballots (match_key), and the
+// column's per-expert running values live in the wavefront's slice of LDS.  Same results as the
+// reference's one-work-item-per-column serial loops, entry for entry.
+constexpr int COL_WAVES = 4;   // columns per block
+
 template <typename TI>
-__global__ void partial_token_counts_kernel(const TI *__restrict__ selected_experts,
-                                            int32_t *__restrict__ partial_token_counts,
-                                            int32_t *__restrict__ expert_counts_ep, int start, int end,
-                                            int K, int64_t TB, int64_t TH) {
-    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (tid >= TH) return;
-    for (int64_t lt = 0; lt < TB; lt++) {
-        int expert_count = 0;
-        const int64_t t = tid * TB + lt;
+__global__ __launch_bounds__(COL_WAVES * 64) void column_counts_kernel(
+    const TI *__restrict__ selected_experts, int32_t *__restrict__ partial_token_counts,
+    int32_t *__restrict__ expert_counts_ep, int start, int end, int NR, int nbits, int K, int64_t TB,
+    int64_t TH) {
+    extern __shared__ int lds[];   // [COL_WAVES][NR]
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t col = static_cast<int64_t>(blockIdx.x) * COL_WAVES + wv;
+    if (col >= TH) return;   // whole wavefronts leave; no block-wide barrier below
+    volatile int *hist = lds + wv * NR;
+    for (int e = lane; e < NR; e += 64) hist[e] = 0;
+    __builtin_amdgcn_wave_barrier();
+    const int64_t j0 = col * TB * K, j1 = j0 + TB * K;
+    for (int64_t base = j0; base < j1; base += 64) {
+        const int key = local_key(selected_experts, base + lane, j1, start, end, NR);
+        const unsigned long long m = match_key(key, nbits);
+        if (key < NR && (__ffsll(static_cast<long long>(m)) - 1) == lane) hist[key] += __popcll(m);
+        __builtin_amdgcn_wave_barrier();
+    }
+    for (int e = lane; e < NR; e += 64) {
+        const int c = hist[e];
+        if (c) partial_token_counts[static_cast<int64_t>(e) * TH + col] += c;   // the table is updated in place
+    }
+    // local hits per token: lanes over the column's tokens
+    for (int64_t t = col * TB + lane; t < (col + 1) * TB; t += 64) {
+        int hits = 0;
         for (int k = 0; k < K; k++) {
-            const long long n = static_cast<long long>(selected_experts[t * K + k]);
-            if (n >= start && n < end) {
-                partial_token_counts[(n - start) * TH + tid] += 1;
-                expert_count += 1;
-            }
+            const long long e = static_cast<long long>(selected_experts[t * K + k]);
+            hits += (e >= start && e < end) ? 1 : 0;
         }
-        expert_counts_ep[t] = expert_count;
+        expert_counts_ep[t] = hits;
     }
 }
 
 template <typename TI>
-__global__ void input_and_output_indices_kernel(
+__global__ __launch_bounds__(COL_WAVES * 64) void column_scatter_kernel(
     const TI *__restrict__ selected_experts, const int32_t *__restrict__ partial_cum_token_counts,
     int32_t *__restrict__ input_increment_buffer, const int32_t *__restrict__ cum_expert_counts_ep,
     int32_t *__restrict__ selected_experts_indices, int32_t *__restrict__ input_indices,
-    int32_t *__restrict__ output_indices, int start, int end, int K, int64_t TB, int64_t TH) {
-    const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (tid >= TH) return;
-    for (int64_t t = tid * TB; t < (tid + 1) * TB; t++) {
-        int output_index = cum_expert_counts_ep[t];
-        for (int k = 0; k < K; k++) {
-            const long long n = static_cast<long long>(selected_experts[t * K + k]);
-            if (n >= start && n < end) {
-                const int64_t cell = (n - start) * TH + tid;
-                const int offset = input_increment_buffer[cell];
-                const int input_index = partial_cum_token_counts[cell] + offset;
-                input_indices[input_index] = static_cast<int32_t>(t);
-                input_increment_buffer[cell] = offset + 1;
-                output_indices[output_index] = input_index;
-                selected_experts_indices[output_index] = k;
-                output_index += 1;
-            }
+    int32_t *__restrict__ output_indices, int start, int end, int NR, int nbits, int K, int64_t TB,
+    int64_t TH) {
+    extern __shared__ int lds[];   // [COL_WAVES][NR]: next free position of every expert in this column
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t col = static_cast<int64_t>(blockIdx.x) * COL_WAVES + wv;
+    if (col >= TH) return;
+    volatile int *off = lds + wv * NR;
+    for (int e = lane; e < NR; e += 64) {
+        const int64_t cell = static_cast<int64_t>(e) * TH + col;
+        off[e] = partial_cum_token_counts[cell] + input_increment_buffer[cell];
+    }
+    __builtin_amdgcn_wave_barrier();
+    const int64_t j0 = col * TB * K, j1 = j0 + TB * K;
+    // kept pairs of the token that straddles into the current 64-pair step
+    int64_t carry_token = -1;
+    int carry_kept = 0;
+    for (int64_t base = j0; base < j1; base += 64) {
+        const int64_t j = base + lane;
+        const bool valid = j < j1;
+        const int key = local_key(selected_experts, j, j1, start, end, NR);
+        const unsigned long long m = match_key(key, nbits);
+        const unsigned long long kept = __ballot(key < NR);
+        const int64_t t = valid ? j / K : -2;
+        const int k = valid ? static_cast<int>(j - t * K) : 0;
+        // lanes of this step that hold earlier pairs of the same token: [first, lane)
+        const int64_t first64 = t * K - base;
+        const int first = first64 > 0 ? static_cast<int>(first64) : 0;
+        const unsigned long long same_before = lanemask_lt(lane) & ~lanemask_lt(first);
+        if (key < NR) {
+            const int oi = cum_expert_counts_ep[t] + __popcll(kept & same_before) +
+                           (t == carry_token ? carry_kept : 0);
+            const int pos = off[key] + __popcll(m & lanemask_lt(lane));
+            input_indices[pos] = static_cast<int32_t>(t);
+            output_indices[oi] = pos;
+            selected_experts_indices[oi] = k;
         }
+        __builtin_amdgcn_wave_barrier();
+        if (key < NR && (__ffsll(static_cast<long long>(m)) - 1) == lane) off[key] += __popcll(m);
+        // the step's last token may continue in the next step: hand its kept pairs on
+        const int64_t t_last = __shfl(t, 63, 64);
+        if (t_last >= 0) {
+            const int here = __popcll(kept & __ballot(t == t_last));
+            carry_kept = (t_last == carry_token ? carry_kept : 0) + here;
+            carry_token = t_last;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    for (int e = lane; e < NR; e += 64) {   // leave the increments as the reference's loop leaves them
+        const int64_t cell = static_cast<int64_t>(e) * TH + col;
+        input_increment_buffer[cell] = off[e] - partial_cum_token_counts[cell];
     }
 }
 
@@ -400,19 +454,22 @@ extern "C" int om_compute_partial_token_counts(const void *selected_experts, int
                                                int expert_end_idx, int64_t T, int K, int64_t TH,
                                                void *stream) {
     if (index_dtype != OM_I32 && index_dtype != OM_I64) return OM_ERR_DTYPE;
-    if (T < 0 || K < 1 || TH < 1 || T % TH != 0) return OM_ERR_SHAPE;
+    const int NR = expert_end_idx - expert_start_idx;
+    if (T < 0 || K < 1 || TH < 1 || T % TH != 0 || NR < 1 || NR > SORT_MAX_NR) return OM_ERR_SHAPE;
     if (T == 0) return OM_OK;
     if (!selected_experts || !partial_token_counts || !expert_counts_ep) return OM_ERR_NULL;
     hipStream_t st = om_stream(stream);
-    const unsigned nb = static_cast<unsigned>((TH + 63) / 64);
+    const unsigned nb = static_cast<unsigned>((TH + COL_WAVES - 1) / COL_WAVES);
+    const size_t lds = static_cast<size_t>(COL_WAVES) * NR * sizeof(int);
+    const int nbits = key_bits(NR);
     if (index_dtype == OM_I64)
-        partial_token_counts_kernel<int64_t><<<nb, 64, 0, st>>>(
+        column_counts_kernel<int64_t><<<nb, COL_WAVES * 64, lds, st>>>(
             static_cast<const int64_t *>(selected_experts), partial_token_counts, expert_counts_ep,
-            expert_start_idx, expert_end_idx, K, T / TH, TH);
+            expert_start_idx, expert_end_idx, NR, nbits, K, T / TH, TH);
     else
-        partial_token_counts_kernel<int32_t><<<nb, 64, 0, st>>>(
+        column_counts_kernel<int32_t><<<nb, COL_WAVES * 64, lds, st>>>(
             static_cast<const int32_t *>(selected_experts), partial_token_counts, expert_counts_ep,
-            expert_start_idx, expert_end_idx, K, T / TH, TH);
+            expert_start_idx, expert_end_idx, NR, nbits, K, T / TH, TH);
     return om_launch_status();
 }
 
@@ -422,22 +479,25 @@ extern "C" int om_compute_input_and_output_indices(
     int32_t *selected_experts_indices, int32_t *input_indices, int32_t *output_indices,
     int expert_start_idx, int expert_end_idx, int64_t T, int K, int64_t TH, void *stream) {
     if (index_dtype != OM_I32 && index_dtype != OM_I64) return OM_ERR_DTYPE;
-    if (T < 0 || K < 1 || TH < 1 || T % TH != 0) return OM_ERR_SHAPE;
+    const int NR = expert_end_idx - expert_start_idx;
+    if (T < 0 || K < 1 || TH < 1 || T % TH != 0 || NR < 1 || NR > SORT_MAX_NR) return OM_ERR_SHAPE;
     if (T == 0) return OM_OK;
     if (!selected_experts || !partial_cum_token_counts || !input_increment_buffer ||
         !cum_expert_counts_ep || !selected_experts_indices || !input_indices || !output_indices)
         return OM_ERR_NULL;
     hipStream_t st = om_stream(stream);
-    const unsigned nb = static_cast<unsigned>((TH + 63) / 64);
+    const unsigned nb = static_cast<unsigned>((TH + COL_WAVES - 1) / COL_WAVES);
+    const size_t lds = static_cast<size_t>(COL_WAVES) * NR * sizeof(int);
+    const int nbits = key_bits(NR);
     if (index_dtype == OM_I64)
-        input_and_output_indices_kernel<int64_t><<<nb, 64, 0, st>>>(
+        column_scatter_kernel<int64_t><<<nb, COL_WAVES * 64, lds, st>>>(
             static_cast<const int64_t *>(selected_experts), partial_cum_token_counts,
             input_increment_buffer, cum_expert_counts_ep, selected_experts_indices, input_indices,
-            output_indices, expert_start_idx, expert_end_idx, K, T / TH, TH);
+            output_indices, expert_start_idx, expert_end_idx, NR, nbits, K, T / TH, TH);
     else
-        input_and_output_indices_kernel<int32_t><<<nb, 64, 0, st>>>(
+        column_scatter_kernel<int32_t><<<nb, COL_WAVES * 64, lds, st>>>(
             static_cast<const int32_t *>(selected_experts), partial_cum_token_counts,
             input_increment_buffer, cum_expert_counts_ep, selected_experts_indices, input_indices,
-            output_indices, expert_start_idx, expert_end_idx, K, T / TH, TH);
+            output_indices, expert_start_idx, expert_end_idx, NR, nbits, K, T / TH, TH);
     return om_launch_status();
 }

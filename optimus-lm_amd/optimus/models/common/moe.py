@@ -72,33 +72,8 @@ def _grouped_gemm(kind, a, b, out, cum, rows, G, N, K, w_stride):
 # ----------------------------------------------------------------------------------------------
 # Router
 # ----------------------------------------------------------------------------------------------
-class Fp32LogitsFunction(torch.autograd.Function):
-    """logits = x.float() @ weight.float().T for bf16 x and weight, without the fp32 copies.
-
-    The products of two bf16 values are exact in fp32, so a bf16 GEMM that accumulates and
-    returns fp32 gives what the fp32 GEMM of the up-cast operands gives, up to the order of the
-    sum (reference: modeling_deepseek_v3.py:160 casts both operands to float32 first).  Backward
-    rounds the logits' gradient to bf16 — the precision a bf16 router's backward has anyway — and
-    runs two bf16 GEMMs; the weight gradient is accumulated and returned from fp32."""
-
-    @staticmethod
-    def forward(ctx, x, weight):
-        ctx.save_for_backward(x, weight)
-        return torch.mm(x, weight.t(), out_dtype=torch.float32)
-
-    @staticmethod
-    def backward(ctx, dlogits):
-        x, weight = ctx.saved_tensors
-        d16 = dlogits.to(torch.bfloat16)
-        dx = torch.mm(d16, weight) if ctx.needs_input_grad[0] else None
-        dw = None
-        if ctx.needs_input_grad[1]:
-            dw = torch.mm(d16.t(), x, out_dtype=torch.float32).to(weight.dtype)
-        return dx, dw
-
-
 def gate_kernel_fits(x, weight):
-    """Shapes and dtypes the fused gate kernels take (om_router_gate_*)."""
+    """Shapes and dtypes the fused gate + routing kernel takes (om_router_gate_softmax_topk)."""
     if not (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
         return False
     N, H = weight.shape
@@ -107,28 +82,19 @@ def gate_kernel_fits(x, weight):
     return H % (512 if N <= 64 else 256 if N <= 128 else 64) == 0
 
 
-def gate_logits_kernel_fits(x, weight):
-    """Shapes and dtypes GateLogitsFunction takes: om_router_gate_logits up to 64 experts,
-    om_router_gate_logits_split above."""
-    if not (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
-        return False
+def _require_gate_shape(weight, h_multiple, what):
     N, H = weight.shape
-    if N > 256 or x.shape[0] == 0:
-        return False
-    return H % (512 if N <= 64 else 64) == 0
-
-
-def gate_wgrad_kernel_fits(x, weight):
-    """Shapes om_router_gate_wgrad takes."""
-    N, H = weight.shape
-    return (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype in (torch.bfloat16, torch.float32)
-            and N in (32, 64, 128, 256) and H % 128 == 0)
+    if N > 256 or H % h_multiple != 0:
+        raise _n.NativeLibraryError(
+            f"{what}: the gate kernels take at most 256 experts and hidden sizes that are multiples "
+            f"of {h_multiple} (got {N} experts, hidden {H}); there is no library fallback")
 
 
 def _gate_weight_grad(x, weight, dlogits):
     """dweight[n,h] = sum_t dlogits[t,n] x[t,h]: a long contraction with a tiny output, split
     over token ranges on the device (om_router_gate_wgrad) instead of a library GEMM that would
     run on a few CUs."""
+    _require_gate_shape(weight, 128, "gate weight gradient")
     T, (N, H) = x.shape[0], weight.shape
     lib = _n.lib()
     ws_bytes = lib.om_router_gate_wgrad_workspace_bytes(T, H, N)
@@ -143,19 +109,34 @@ def _gate_weight_grad(x, weight, dlogits):
     return dw
 
 
-def _gate_backward(x, weight, dlogits, needs):
-    """(dx, dweight) of logits = x @ weight.T from the fp32 gradient of the logits, rounded to
-    bf16 (the precision a bf16 router's backward has anyway): dx by a library GEMM, the weight
-    gradient accumulated in fp32 by om_router_gate_wgrad (a library GEMM for shapes it does not
-    take)."""
+def _gate_input_grad(weight, dlogits, other_grad=None):
+    """dx = bf16(dlogits) @ weight (om_router_gate_dgrad).  With `other_grad` [T,H] (the gradient
+    that reached the same hidden states through the experts) the sum of the two is returned, formed
+    inside the kernel with autograd's two roundings, so no separate accumulation pass runs."""
+    _require_gate_shape(weight, 8, "gate input gradient")
+    T, (N, H) = dlogits.shape[0], weight.shape
+    dlogits = dlogits.contiguous()
+    if other_grad is not None:
+        other_grad = other_grad.contiguous()
+        _require_bf16(other_grad)
+    dx = torch.empty((T, H), dtype=torch.bfloat16, device=dlogits.device)
+    _n.check(_n.lib().om_router_gate_dgrad(_n.ptr(dlogits), _n.ptr(weight), _n.ptr(other_grad), _n.ptr(dx),
+                                           T, H, N, _n.stream()), "om_router_gate_dgrad")
+    return dx
+
+
+def _gate_backward(x, weight, dlogits, needs, other_grad=None):
+    """(dx, dweight) of logits = x @ weight.T for a bf16 gate from the fp32 gradient of the logits,
+    rounded to bf16 as it is loaded (the precision a bf16 router's backward has anyway), both on
+    bf16 MFMA with fp32 accumulation: om_router_gate_dgrad and om_router_gate_wgrad.  `other_grad`
+    is added to dx inside the kernel (see _gate_input_grad)."""
+    _require_bf16(x, weight)
+    dlogits = dlogits.to(torch.float32)
     dx = dw = None
     if needs[0]:
-        dx = torch.mm(dlogits.to(torch.bfloat16), weight)
+        dx = _gate_input_grad(weight, dlogits, other_grad)
     if needs[1]:
-        if gate_wgrad_kernel_fits(x, weight) and dlogits.dtype == torch.float32:
-            dw = _gate_weight_grad(x, weight, dlogits)
-        else:
-            dw = torch.mm(dlogits.to(torch.bfloat16).t(), x, out_dtype=torch.float32).to(weight.dtype)
+        dw = _gate_weight_grad(x, weight, dlogits)
     return dx, dw
 
 
@@ -167,8 +148,9 @@ class GateLogitsFunction(torch.autograd.Function):
         T, (N, H) = x.shape[0], weight.shape
         logits = torch.empty((T, N), dtype=torch.float32, device=x.device)
         lib = _n.lib()
-        if N > 64 and H % 64 == 0:
+        if N > 64 or H % 512 != 0:
             # many experts: the weight no longer fits a block's re-reads; split over H instead
+            # (also the form for hidden sizes the one-pass kernel does not take)
             ws_bytes = lib.om_router_gate_logits_split_workspace_bytes(T, H, N)
             if ws_bytes < 0:
                 _n.check(int(ws_bytes), "om_router_gate_logits_split_workspace_bytes")
@@ -189,18 +171,38 @@ class GateLogitsFunction(torch.autograd.Function):
 
 
 def fp32_logits(x, weight):
-    """Router logits in float32 from 2-D x [T,H] and weight [N,H] (the gate's nn.Linear weight)."""
-    if gate_logits_kernel_fits(x, weight):
+    """Router logits in float32 from 2-D x [T,H] and weight [N,H] (the gate's nn.Linear weight).
+    bf16 operands go through the gate kernels (at most 256 experts, H a multiple of 64; anything
+    else raises); a float32 module's gate is torch's own float32 linear."""
+    if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
+        _n.require_cuda_contiguous(x.contiguous(), weight.contiguous())
+        _require_gate_shape(weight, 64, "gate projection")
         return GateLogitsFunction.apply(x.contiguous(), weight.contiguous())
-    if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.is_cuda:
-        return Fp32LogitsFunction.apply(x.contiguous(), weight.contiguous())
-    return torch.nn.functional.linear(x.float(), weight.float())
+    if x.dtype == torch.float32 and weight.dtype == torch.float32:
+        return torch.nn.functional.linear(x, weight)
+    raise TypeError(f"router gate: activations and weight must both be bfloat16 or both float32 "
+                    f"(got {x.dtype}, {weight.dtype})")
+
+
+def gate_logits(x, gate):
+    """router_logits = gate(x) in the module's dtype (reference moe.py:456,
+    modeling_olmoe.py:284) for 2-D x.  A bf16 gate runs on the gate kernels: the fp32-accumulated
+    logits rounded once to bf16, which is what a bf16 linear layer returns (up to the order of the
+    fp32 sum).  A float32 module's gate is torch's own float32 linear."""
+    if x.dtype == torch.bfloat16 and gate.weight.dtype == torch.bfloat16:
+        return fp32_logits(x, gate.weight).to(torch.bfloat16)
+    return gate(x)
 
 
 class GateSoftmaxTopkFunction(torch.autograd.Function):
     """The OLMoE router in one launch (om_router_gate_softmax_topk): gate projection with fp32
     logits, softmax, top-K, optional renormalisation.  Returns (routing_weights, selected_experts,
-    router_logits fp32); reference moe.py:456 and :467-471."""
+    router_logits fp32, hidden_states); reference moe.py:456 and :467-471.
+
+    The fourth output is the input itself.  A caller that feeds the experts from it (instead of from
+    the tensor it passed in) makes the experts' input gradient arrive here, where the gate's own
+    input gradient is added to it inside om_router_gate_dgrad: one pass over [T,H] instead of a
+    matmul output plus autograd's accumulation kernel."""
 
     @staticmethod
     def forward(ctx, x, weight, top_k, norm_topk_prob, out_dtype):
@@ -219,15 +221,15 @@ class GateSoftmaxTopkFunction(torch.autograd.Function):
         # an output nobody differentiates (the logits without an auxiliary loss) arrives as None in
         # backward instead of a tensor of zeros that would have to be filled and added
         ctx.set_materialize_grads(False)
-        return weights, experts, logits
+        return weights, experts, logits, x.view_as(x)
 
     @staticmethod
-    def backward(ctx, weights_grad, _experts_grad, logits_grad):
+    def backward(ctx, weights_grad, _experts_grad, logits_grad, x_grad):
         x, weight, logits, experts = ctx.saved_tensors
         T, N = logits.shape
         K = experts.shape[1]
         if weights_grad is None and logits_grad is None:
-            return None, None, None, None, None
+            return x_grad, None, None, None, None
         if weights_grad is None:
             dlogits = logits_grad.to(torch.float32).contiguous()
         else:
@@ -239,7 +241,7 @@ class GateSoftmaxTopkFunction(torch.autograd.Function):
                 _n.stream()), "om_route_softmax_topk_bwd")
             if logits_grad is not None:
                 dlogits = dlogits + logits_grad
-        dx, dw = _gate_backward(x, weight, dlogits, ctx.needs_input_grad)
+        dx, dw = _gate_backward(x, weight, dlogits, ctx.needs_input_grad, other_grad=x_grad)
         return dx, dw, None, None, None
 
 
@@ -1058,14 +1060,17 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
         flat = hidden_states.reshape(-1, hidden_dim)
         if self.router_logits_fp32 and gate_kernel_fits(flat, self.gate.weight):
-            routing_weights, selected_experts, router_logits = GateSoftmaxTopkFunction.apply(
+            # the experts read the router function's pass-through of the hidden states, so that their
+            # input gradient and the gate's are added in one kernel (GateSoftmaxTopkFunction)
+            routing_weights, selected_experts, router_logits, flat = GateSoftmaxTopkFunction.apply(
                 flat.contiguous(), self.gate.weight, self.num_experts_per_tok, self.norm_topk_prob,
                 hidden_states.dtype)
+            hidden_states = flat.view(batch_size, sequence_length, hidden_dim)
         else:
             if self.router_logits_fp32:
                 router_logits = fp32_logits(flat, self.gate.weight)
             else:
-                router_logits = self.gate(flat)
+                router_logits = gate_logits(flat, self.gate)
             routing_weights, selected_experts = SoftmaxTopkRouterFunction.apply(
                 router_logits.contiguous(), self.num_experts_per_tok, self.norm_topk_prob,
                 hidden_states.dtype)

@@ -81,7 +81,7 @@ class OlmoeParallelSparseMoeBlock(nn.Module):
 
     def forward(self, hidden_states):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
-        router_logits = self.gate(hidden_states.reshape(-1, hidden_dim))
+        router_logits = _moe.gate_logits(hidden_states.reshape(-1, hidden_dim), self.gate)
         routing_weights, selected_experts = _moe.SoftmaxTopkRouterFunction.apply(
             router_logits.contiguous(), self.num_experts_per_tok, self.norm_topk_prob,
             hidden_states.dtype)

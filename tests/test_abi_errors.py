@@ -72,9 +72,20 @@ def test_routers(lib):
     need = lib.om_router_gate_wgrad_workspace_bytes(16384, 2048, 64)
     assert need > 0 and need % 16 == 0
     assert lib.om_router_gate_wgrad_workspace_bytes(16384, 2000, 64) == SHAPE      # H % 128
-    assert lib.om_router_gate_wgrad_workspace_bytes(16384, 2048, 48) == SHAPE      # N not 32/64/128/256
+    assert lib.om_router_gate_wgrad_workspace_bytes(16384, 2048, 300) == SHAPE     # more than 256 experts
+    assert lib.om_router_gate_wgrad_workspace_bytes(16384, 2048, 48) > 0           # any expert count up to 256
     assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 64, P, 7, P, need, None) == DTYPE
-    assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 96, P, BF16, P, need, None) == SHAPE
+    assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 0, P, BF16, P, need, None) == SHAPE
+    assert lib.om_router_gate_dgrad(P, P, None, P, 16384, 2044, 64, None) == SHAPE      # H % 8
+    assert lib.om_router_gate_dgrad(P, P, None, P, 16384, 2048, 257, None) == SHAPE
+    assert lib.om_router_gate_dgrad(P, None, None, P, 16384, 2048, 64, None) == NULL
+    assert lib.om_router_gate_dgrad(P, P, ODD, P, 16384, 2048, 64, None) == ALIGN
+    assert lib.om_router_gate_dgrad(None, None, None, None, 0, 2048, 64, None) == OK
+    assert lib.om_grad_scale(P, 100, 7, P, None) == DTYPE
+    assert lib.om_grad_scale(P, 100, BF16, None, None) == NULL
+    assert lib.om_grad_scale(ODD, 100, BF16, P, None) == ALIGN
+    assert lib.om_grad_scale(None, 0, BF16, None, None) == OK
+    assert lib.om_adamw_traffic_probe(P, P, P, None, P, 1024, None) == NULL
     assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 64, None, BF16, P, need, None) == NULL
     assert lib.om_router_gate_wgrad(P, None, 16384, 2048, 64, P, BF16, P, need, None) == NULL
     assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 64, ODD, BF16, P, need, None) == ALIGN
@@ -128,7 +139,8 @@ def test_grouped_gemms(lib):
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 4096, 1025, 256, 256, 0, None) == SHAPE      # G > 1024 (LDS table)
     assert lib.om_grouped_gemm_fwd(P, None, P, P, *args) == NULL
     assert lib.om_grouped_gemm_fwd(P, P, ODD, P, *args) == ALIGN
-    assert lib.om_grouped_gemm_fwd(P, P, P, P, 1 << 22, 64, 2048, 1024, 0, None) == SHAPE   # > 2^31 elements
+    assert lib.om_grouped_gemm_fwd(P, P, P, P, 1 << 25, 64, 2048, 1024, 0, None) == SHAPE   # 2^35 elements or more
+    assert lib.om_grouped_gemm_fwd(P, P, P, P, 4096, 64, 2048, 1024, 2048 * 1024 + 4, None) == ALIGN   # expert pitch % 8
     assert lib.om_grouped_gemm_dgrad(P, P, P, None, *args) == NULL
     assert lib.om_grouped_gemm_wgrad(P, P, P, P, 131072, 0, 2048, 1024, 0, None) == SHAPE   # G < 1
     assert lib.om_merged_mlp_gate_up_fwd(P, P, P, P, P, P, P, 131072, 64, 1000, 2048, 0, None) == SHAPE
@@ -147,7 +159,7 @@ def test_grouped_gemms(lib):
     g = (131072, 64, 1024, 2048, 0, None)
     assert lib.om_merged_mlp_gate_up_fwd_gathered(P, None, 16384, P, P, P, P, P, P, *g) == NULL      # no index
     assert lib.om_merged_mlp_gate_up_fwd_gathered(P, P, 0, P, P, P, P, P, P, *g) == SHAPE            # no source rows
-    assert lib.om_merged_mlp_gate_up_fwd_gathered(P, P, 1 << 21, P, P, P, P, P, P, *g) == SHAPE      # source > 2^31 elements
+    assert lib.om_merged_mlp_gate_up_fwd_gathered(P, P, 1 << 24, P, P, P, P, P, P, *g) == SHAPE      # source of 2^35 elements or more
     assert lib.om_merged_mlp_gate_up_fwd_gathered(P, None, 0, P, P, P, P, P, P, 0, 64, 1024, 2048, 0, None) == OK
     assert lib.om_grouped_gemm_wgrad_gathered(P, P, None, 16384, P, P, *g) == NULL
     assert lib.om_grouped_gemm_wgrad_gathered(P, P, P, 0, P, P, *g) == SHAPE
@@ -171,7 +183,7 @@ def test_routing_weight_folded_into_the_expert_mlp(lib):
     gw = (131072, 64, 2048, 1024, 0, None)
     assert lib.om_grouped_gemm_wgrad_gathered_out(P, None, 16384, P, P, P, *gw) == NULL
     assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 0, P, P, P, *gw) == SHAPE
-    assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 1 << 21, P, P, P, *gw) == SHAPE   # source > 2^31 elements
+    assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 1 << 25, P, P, P, *gw) == SHAPE   # source of 2^35 elements or more
     assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 16384, P, ODD, P, *gw) == ALIGN
     assert lib.om_merged_mlp_row_dot_parts(1024) == 16
     assert lib.om_merged_mlp_row_dot_parts(100) == SHAPE

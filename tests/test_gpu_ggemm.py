@@ -324,3 +324,44 @@ def test_wgrad_with_thousands_of_experts(cuda, G, rows, N, K):
         ref[e] = dy[s:t].float().t() @ x[s:t].float()
     assert max_abs(got, ref) <= 1e-2 * max(1.0, float(ref.abs().max()))
     assert float(got[c == 0].abs().max()) == 0.0
+
+
+def test_operands_beyond_2_31_elements(cuda):
+    """Activations of 1.1M rows x 2048 (2.25e9 elements, 4.5 GB): every product of the merged MLP,
+    forward and backward, reads or writes a tensor past the 2^31-element mark.  Rows at the start,
+    around the mark and at the end are checked against fp32 per-expert products, and so are the
+    weight gradients of the expert whose rows straddle the mark and of the last one."""
+    from optimus.models.common.moe import MergedMLPFunction
+    rows, H, I, G = 1_100_000, 2048, 128, 4
+    assert rows * H > (1 << 31)
+    cum = torch.tensor([0, 500_000, 1_000_000, 1_099_000, rows], dtype=torch.int32)
+    gen = torch.Generator(device=cuda).manual_seed(77)
+    x = torch.randn(rows, H, device=cuda, dtype=torch.bfloat16, generator=gen).requires_grad_(True)
+    dy = torch.randn(rows, H, device=cuda, dtype=torch.bfloat16, generator=gen)
+    ws = [(torch.randn(shape, device=cuda, dtype=torch.float32, generator=gen) * 0.03).to(torch.bfloat16).requires_grad_(True)
+          for shape in ((G, I, H), (G, I, H), (G, H, I))]
+    y = MergedMLPFunction.apply(x, *ws, cum.to(cuda))
+    y.backward(dy)
+    torch.cuda.synchronize()
+    mark = (1 << 31) // H
+    picks = torch.cat([torch.arange(0, 48), torch.arange(mark - 40, mark + 40), torch.arange(999_980, 1_000_020),
+                       torch.arange(rows - 48, rows)])
+    expert_of = torch.bucketize(picks, cum[1:].long(), right=True)
+    wf = [w.detach().float().cpu() for w in ws]
+    for e in range(G):
+        sel = picks[expert_of == e]
+        if sel.numel() == 0:
+            continue
+        xr = x.detach()[sel.to(cuda)].float().cpu().requires_grad_(True)
+        yr = (torch.nn.functional.silu(xr @ wf[0][e].t()) * (xr @ wf[1][e].t())) @ wf[2][e].t()
+        yr.backward(dy[sel.to(cuda)].float().cpu())
+        assert_bf16_parity(y.detach()[sel.to(cuda)], yr, *MLP_BARS["out"], tag=f"beyond2^31 expert {e} y")
+        assert_bf16_parity(x.grad[sel.to(cuda)], xr.grad, *MLP_BARS["grad"], tag=f"beyond2^31 expert {e} dx")
+    for e in (2, 3):       # rows 1,000,000..1,099,000 straddle the mark; 1,099,000.. lie beyond it
+        s0, s1 = int(cum[e]), int(cum[e + 1])
+        xr = x.detach()[s0:s1].float().cpu()
+        p = [w[e].clone().requires_grad_(True) for w in wf]
+        yr = (torch.nn.functional.silu(xr @ p[0].t()) * (xr @ p[1].t())) @ p[2].t()
+        yr.backward(dy[s0:s1].float().cpu())
+        for name, w, r in zip(("dwg", "dwu", "dwd"), ws, p):
+            assert_bf16_parity(w.grad[e], r.grad, *MLP_BARS["grad"], tag=f"beyond2^31 expert {e} {name}")

@@ -180,7 +180,7 @@ def _gate_inputs(T, H, N, seed):
 
 
 @pytest.mark.parametrize("T,H,N", [(1000, 2048, 64), (64, 512, 8), (33, 1024, 128), (300, 7168, 256),
-                                   (4096, 2048, 60),
+                                   (4096, 2048, 60), (200, 2304, 8), (77, 192, 60),   # hidden sizes the one-pass kernel does not take
                                    # more than 64 experts: the kernel that shares the weight tile
                                    # through LDS and splits H (odd step counts, padded expert rows,
                                    # a partial last 128-token block, one and several slices)
@@ -188,9 +188,8 @@ def _gate_inputs(T, H, N, seed):
 def test_gate_logits_match_fp32_matmul(cuda, T, H, N):
     """fp32 logits from bf16 operands: the products are exact, only the order of the fp32 sum differs
     from the CPU matmul of the up-cast operands."""
-    from optimus.models.common.moe import fp32_logits, gate_logits_kernel_fits
+    from optimus.models.common.moe import fp32_logits
     x, w = _gate_inputs(T, H, N, seed=T + N)
-    assert gate_logits_kernel_fits(x.to(cuda), w.to(cuda))
     got = fp32_logits(x.to(cuda), w.to(cuda)).cpu()
     ref = x.float() @ w.float().t()
     exact = (x.double() @ w.double().t())
@@ -212,7 +211,8 @@ def test_gate_softmax_topk_equals_two_step_on_its_own_logits(cuda, T, H, N, K, r
     equal the CPU oracle's on rows without near-ties."""
     from optimus.models.common.moe import GateSoftmaxTopkFunction, SoftmaxTopkRouterFunction
     x, w = _gate_inputs(T, H, N, seed=7 * T + N)
-    wts, exp, logits = GateSoftmaxTopkFunction.apply(x.to(cuda), w.to(cuda), K, renorm, wdt)
+    wts, exp, logits, x_out = GateSoftmaxTopkFunction.apply(x.to(cuda), w.to(cuda), K, renorm, wdt)
+    assert x_out.data_ptr() != 0 and torch.equal(x_out.cpu(), x)      # the pass-through of the hidden states
     w2, e2 = SoftmaxTopkRouterFunction.apply(logits.contiguous(), K, renorm, wdt)
     assert torch.equal(exp, e2) and torch.equal(wts.view(torch.int16 if wdt == torch.bfloat16 else torch.int32),
                                                 w2.view(torch.int16 if wdt == torch.bfloat16 else torch.int32))
@@ -234,11 +234,12 @@ def test_gate_softmax_topk_backward(cuda):
     dw_out = torch.randn(T, K, generator=g)
     dlogit_out = torch.randn(T, N, generator=g) * 0.1
     xg = x.to(cuda).requires_grad_(True); wg = w.to(cuda).requires_grad_(True)
-    wts, exp, logits = GateSoftmaxTopkFunction.apply(xg, wg, K, True, torch.float32)
+    dx_other = torch.randn(T, H, generator=g).to(torch.bfloat16)     # a gradient arriving through the pass-through
+    wts, exp, logits, x_out = GateSoftmaxTopkFunction.apply(xg, wg, K, True, torch.float32)
     (wts * dw_out.to(cuda)).sum().backward(retain_graph=True)
     gx1, gw1 = xg.grad.clone(), wg.grad.clone()
     xg.grad = None; wg.grad = None
-    ((wts * dw_out.to(cuda)).sum() + (logits * dlogit_out.to(cuda)).sum()).backward()
+    ((wts * dw_out.to(cuda)).sum() + (logits * dlogit_out.to(cuda)).sum()).backward(retain_graph=True)
     # reference in fp32 on the CPU with the kernel's own expert choice
     xr = x.float().requires_grad_(True); wr = w.float().requires_grad_(True)
     lr = xr @ wr.t()
@@ -248,22 +249,32 @@ def test_gate_softmax_topk_backward(cuda):
     rel = lambda a, b: float((a.float().cpu() - b).abs().mean() / b.abs().mean())
     assert rel(xg.grad, xr.grad) < 1e-2 and rel(wg.grad, wr.grad) < 1e-2
     assert not torch.equal(gx1, xg.grad)     # the logits' own gradient takes part
+    # a gradient through the pass-through output is added inside the kernel with autograd's two
+    # roundings: bf16(float(other) + float(gate dx)) bit for bit
+    gate_dx = xg.grad.clone()
+    xg.grad = None; wg.grad = None
+    ((wts * dw_out.to(cuda)).sum() + (logits * dlogit_out.to(cuda)).sum()
+     + (x_out.float() * dx_other.to(cuda).float()).sum()).backward()
+    want = (dx_other.to(cuda).float() + gate_dx.float()).to(torch.bfloat16)
+    assert torch.equal(xg.grad, want)
 
 
 @pytest.mark.parametrize("T,H,N,wdt", [(16384, 2048, 64, torch.bfloat16), (1, 128, 32, torch.float32),
                                        (100, 256, 64, torch.float32), (5000, 1024, 128, torch.bfloat16),
-                                       (777, 7168, 256, torch.float32), (64, 2048, 64, torch.float32)])
+                                       (777, 7168, 256, torch.float32), (64, 2048, 64, torch.float32),
+                                       # expert counts that are no multiple of 32 or of 4
+                                       (300, 256, 8, torch.bfloat16), (1000, 384, 60, torch.float32),
+                                       (500, 128, 130, torch.float32), (257, 512, 7, torch.float32)])
 def test_gate_weight_grad_matches_fp32_matmul(cuda, T, H, N, wdt):
     """om_router_gate_wgrad against the product it replaces: dlogits rounded to bf16, multiplied in
     fp32.  The bf16 x bf16 products are exact in fp32, so only the order of the fp32 sum differs
     (float64 reference; bound = a few fp32 roundings of the absolute sum), plus one final rounding
     for a bf16 weight.  Token counts that are not multiples of the 64-token stage or of the split."""
-    from optimus.models.common.moe import _gate_weight_grad, gate_wgrad_kernel_fits
+    from optimus.models.common.moe import _gate_weight_grad
     g = torch.Generator().manual_seed(T + N)
     x = torch.randn(T, H, generator=g).to(torch.bfloat16)
     dl = torch.randn(T, N, generator=g) * 0.3
     w = torch.empty(N, H, dtype=wdt)
-    assert gate_wgrad_kernel_fits(x.to(cuda), w.to(cuda))
     out = _gate_weight_grad(x.to(cuda), w.to(cuda), dl.to(cuda))
     assert out.dtype == wdt and out.shape == (N, H)
     d16 = dl.to(torch.bfloat16).double()
@@ -312,3 +323,52 @@ def test_balance_loss_gradient_and_bf16_logits(cuda):
     got = float(load_balancing_loss_func(tuple(l.to(cuda) for l in b16), N, K))
     want = float(R.load_balancing_loss(tuple(l.float() for l in b16), N, K))
     assert abs(got - want) <= 1e-3 * want
+
+
+@pytest.mark.parametrize("T,H,N,with_other", [(16384, 2048, 64, True), (1, 128, 32, False), (100, 264, 60, True),
+                                              (5000, 1024, 128, False), (777, 7168, 256, True), (130, 2304, 7, True),
+                                              (64, 8, 5, False)])
+def test_gate_input_grad_matches_fp32_matmul(cuda, T, H, N, with_other):
+    """om_router_gate_dgrad against the product it replaces, mm(bf16(dlogits), W): exact products,
+    fp32 sums in another order, one bf16 rounding; with `other` the second rounding of the
+    accumulation.  Partial token blocks, partial column blocks, expert counts that need padding."""
+    from optimus.models.common.moe import _gate_input_grad
+    g = torch.Generator().manual_seed(3 * T + N)
+    w = (torch.randn(N, H, generator=g) * 0.05).to(torch.bfloat16)
+    dl = torch.randn(T, N, generator=g) * 0.3
+    other = torch.randn(T, H, generator=g).to(torch.bfloat16) if with_other else None
+    got = _gate_input_grad(w.to(cuda), dl.to(cuda), None if other is None else other.to(cuda))
+    assert got.dtype == torch.bfloat16 and got.shape == (T, H)
+    d16 = dl.to(torch.bfloat16).double()
+    exact = d16 @ w.double()
+    bound = 1e-6 * (d16.abs() @ w.double().abs()) + exact.abs() * 2.0 ** -8 + 1e-30     # order of the sum + one rounding
+    if other is None:
+        err = (got.double().cpu() - exact).abs()
+        assert bool((err <= bound).all()), float((err / bound).max())
+    else:
+        total = other.double() + exact
+        err = (got.double().cpu() - total).abs()
+        bound = bound + total.abs() * 2.0 ** -8
+        assert bool((err <= bound).all()), float((err / bound).max())
+        # exactly the two roundings: round the kernel's own product, add, round
+        alone = _gate_input_grad(w.to(cuda), dl.to(cuda))
+        assert torch.equal(got, (other.to(cuda).float() + alone.float()).to(torch.bfloat16))
+    assert torch.equal(got, _gate_input_grad(w.to(cuda), dl.to(cuda), None if other is None else other.to(cuda)))
+
+
+def test_gate_shapes_without_a_kernel_raise(cuda):
+    """No library fallback behind the gate: a bf16 gate whose shape the kernels do not take raises."""
+    from optimus._native import NativeLibraryError
+    from optimus.models.common.moe import _gate_backward, fp32_logits
+    x = torch.zeros(16, 100, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(NativeLibraryError):
+        fp32_logits(x, torch.zeros(8, 100, dtype=torch.bfloat16, device=cuda))            # H % 64
+    x = torch.zeros(16, 128, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(NativeLibraryError):
+        fp32_logits(x, torch.zeros(300, 128, dtype=torch.bfloat16, device=cuda))          # more than 256 experts
+    x = torch.zeros(16, 192, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(NativeLibraryError):
+        _gate_backward(x, torch.zeros(8, 192, dtype=torch.bfloat16, device=cuda),
+                       torch.zeros(16, 8, device=cuda), (False, True))                      # weight gradient: H % 128
+    with pytest.raises(TypeError):
+        fp32_logits(x, torch.zeros(8, 192, dtype=torch.float32, device=cuda))              # mixed dtypes

@@ -63,14 +63,21 @@ def test_permutation_invariants_full_size(cuda):
     assert np.array_equal(np.bincount(se.numpy().reshape(-1), minlength=N), np.diff(cum))
 
 
-@pytest.mark.parametrize("T,N,K,start,end", [(2048, 8, 2, 0, 8), (4096, 64, 8, 16, 48)])
-def test_reference_shaped_index_ops(cuda, oracle_lib, T, N, K, start, end):
+@pytest.mark.parametrize("T,N,K,start,end,TB", [
+    (2048, 8, 2, 0, 8, 8), (4096, 64, 8, 16, 48, 8),     # the reference's blocking: 8 tokens per column
+    (1536, 16, 3, 0, 16, 32),      # 96 pairs per column: two 64-pair steps, a token straddles them
+    (640, 300, 5, 20, 290, 64),    # 320 pairs per column, five steps, more than 256 local experts
+    (77, 8, 2, 2, 6, 1),           # one token per column
+    (512, 64, 8, 0, 64, 512),      # a single column holds every token
+])
+def test_reference_shaped_index_ops(cuda, oracle_lib, T, N, K, start, end, TB):
     """pcl_xpu_customops.compute_partial_token_counts / compute_input_and_output_indices with the
-    reference's own call sequence (moe.py:492-554), torch.cumsum as K2."""
+    reference's own call sequence (moe.py:492-554), torch.cumsum as K2; the table has one column per
+    TB consecutive tokens (the reference fixes TB = 8, the operators take any T / TH)."""
     import pcl_xpu_customops as ops
-    se = routed_experts(T, N, K, seed=11).to(cuda)
-    NR, TH = end - start, T // 8
-    ref = oracle_lib.index_construction(se.cpu().numpy(), NR, start, end)
+    se = routed_experts(T, N, K, seed=11, skew=0.7).to(cuda)
+    NR, TH = end - start, T // TB
+    ref = oracle_lib.index_construction(se.cpu().numpy(), NR, start, end, tokens_per_thread=TB)
     i32 = dict(dtype=torch.int32, device=cuda)
     partial = torch.zeros((NR, TH), **i32)
     partial_cum = torch.zeros(NR * TH + 1, **i32)
@@ -90,6 +97,8 @@ def test_reference_shaped_index_ops(cuda, oracle_lib, T, N, K, start, end):
     assert np.array_equal(ii.cpu().numpy(), ref["input_indices"])
     assert np.array_equal(oi.cpu().numpy(), ref["output_indices"])
     assert np.array_equal(si.cpu().numpy(), ref["selected_experts_indices"])
+    # the increments end as the per-column counts, like the reference's read-modify-write leaves them
+    assert np.array_equal(incr.cpu().numpy(), ref["partial_token_counts"])
 
 
 @pytest.mark.parametrize("seed", list(range(16)))
