@@ -164,6 +164,173 @@ def bench_moe(args, device):
     return dict(T=T, ms_per_step=ms_per_step, roofline=roofline, kernels=kernels, cfg=c)
 
 
+def _timed_steps(step, warmup, steps):
+    """(ms per step by the host clock, {entry point: summed ms over the steps}) for `steps` calls of
+    step() with every C-ABI launch bracketed by HIP events."""
+    import torch
+    from optimus import _native
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    _native.launch_log = []
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    log, _native.launch_log = _native.launch_log, None
+    per = {}
+    for name, a, b in log:
+        per[name] = per.get(name, 0.0) + a.elapsed_time(b)
+    return ms, {k: v / steps for k, v in per.items()}
+
+
+def bench_other_configs(args, device, with_cpu):
+    """The other MoE configurations of BASELINE.json, each as whole-block forward+backward on the GPU:
+    C1 (tiny, run in bf16 here; its float32 CPU reference path timed in full beside it), C4 (skewed
+    small batch on injected router logits) and C5 (one rank's share of a DeepSeek-V3 layer).  For the
+    two whose experts hold few rows (C4, the routed part of C5) the expert GEMMs are bound by
+    streaming the expert weights, so both figures are given: MFMA fraction of the algorithmic flops
+    and weight bytes per second (forward reads every local expert's three matrices once, the input
+    gradients read them once more, the weight gradients write three matrices of the same size)."""
+    import torch
+    import synthetic_configs as sc
+    from optimus.mapper import ParallelDpPpEpTpMapper
+    from optimus.models.common.moe import (MergedMLPFunction, RoutedMLPFunction, SoftmaxTopkRouterFunction,
+                                           expert_computation)
+    steps = max(3, min(args.steps, 10))
+    out = {}
+
+    def gemm_ms(per):
+        return sum(v for k, v in per.items() if k in GEMM_ENTRY_PRODUCTS)
+
+    def entry(T, ms, per, flops, weight_bytes=None, extra=None):
+        g = gemm_ms(per)
+        e = {"ms_per_step": round(ms, 4), "tokens_per_s": round(T / (ms * 1e-3), 1),
+             "expert_gemm_ms": round(g, 4), "expert_gemm_flops": flops,
+             "mfma_frac": round(flops / (g * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+        if weight_bytes is not None:
+            e["weight_stream_gb_per_s"] = round(weight_bytes / (g * 1e-3) / 1e9, 1)
+            e["weight_stream_hbm_frac"] = round(weight_bytes / (g * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
+            e["weight_bytes_per_step"] = weight_bytes
+        if extra:
+            e.update(extra)
+        return e
+
+    # ---- C1 -----------------------------------------------------------------------------------
+    inp = sc.moe_inputs("C1")
+    c = inp["cfg"]
+    blk = build_block(inp, device)
+    x = inp["x"].to(device).view(1, c["T"], c["H"]).requires_grad_(True)
+    dout = inp["dout"].to(device).view_as(x)
+
+    def step_c1():
+        for p in blk.parameters():
+            p.grad = None
+        x.grad = None
+        o, _ = blk(x)
+        o.backward(dout)
+    ms, per = _timed_steps(step_c1, args.warmup, steps)
+    flops = 18.0 * c["T"] * c["K"] * c["H"] * c["I"]
+    out["C1"] = entry(c["T"], ms, per, flops, extra={
+        "workload": "C1 tiny MoE layer fwd+bwd (2048 tokens, hidden 256, 8 experts, top-2 renormalised, ffn 512), "
+                    "bf16 on the GPU; about 25 launches, launch-bound"})
+    if with_cpu:
+        from oracle import moe_layer as L
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        torch.set_num_threads(cores)
+        t = {k: inp[k].float().requires_grad_(True) for k in ("x", "gate_w", "w_gate", "w_up", "w_down")}
+        best = None
+        for _ in range(3):
+            for v in t.values():
+                v.grad = None
+            t0 = time.perf_counter()
+            o, _ = L.olmoe_slow_block(t["x"], t["gate_w"], t["w_gate"], t["w_up"], t["w_down"], c["K"], True)
+            o.backward(inp["dout"].float())
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        out["C1"]["cpu_baseline"] = {"value": round(c["T"] / best, 1), "unit": "tokens/s", "cores": cores,
+                                     "kind": "port", "sample": f"all 2048 tokens, float32, best of 3 ({best * 1e3:.1f} ms)"}
+    del blk, x, dout
+
+    # ---- C4 -----------------------------------------------------------------------------------
+    inp = sc.moe_inputs("C4")
+    c = inp["cfg"]
+    logits = inp["logits"].to(device)
+    t = {k: inp[k].to(device).requires_grad_(True) for k in ("x", "w_gate", "w_up", "w_down")}
+    dout = inp["dout"].to(device)
+    routed = lambda hs, rw, ii, cum_ep, oi, si, cum, res: RoutedMLPFunction.apply(
+        hs, rw, ii, cum_ep, oi, si, cum, res, True, t["w_gate"], t["w_up"], t["w_down"])
+    fn = lambda gi, cum: MergedMLPFunction.apply(gi, t["w_gate"], t["w_up"], t["w_down"], cum)
+
+    def step_c4():
+        for v in t.values():
+            v.grad = None
+        w, e = SoftmaxTopkRouterFunction.apply(logits, c["K"], False, torch.bfloat16)
+        o = expert_computation(t["x"], w.detach().requires_grad_(True), e, 0, c["N"], fn, c["N"],
+                               routed_experts_fn=routed)
+        o.backward(dout)
+    ms, per = _timed_steps(step_c4, args.warmup, steps)
+    flops = 18.0 * c["T"] * c["K"] * c["H"] * c["I"]
+    wbytes = 3 * 3 * c["N"] * c["H"] * c["I"] * 2
+    with torch.no_grad():
+        _, e = SoftmaxTopkRouterFunction.apply(logits, c["K"], False, torch.bfloat16)
+        counts = torch.bincount(e.flatten(), minlength=c["N"])
+    out["C4"] = entry(c["T"], ms, per, flops, wbytes, extra={
+        "workload": "C4 OLMoE-shape layer under Zipf(1.2) routing, 512 tokens (router on injected logits, "
+                    "permutation, expert GEMMs, combine; fwd+bwd)",
+        "rows_per_expert": {"min": int(counts.min()), "median": int(counts.median()), "max": int(counts.max()),
+                            "experts_with_at_most_8_rows": int((counts <= 8).sum())}})
+    del t, logits, dout
+
+    # ---- C5 -----------------------------------------------------------------------------------
+    from optimus.models.deepseek_v3.configuration_deepseek_v3 import DeepseekV3ParallelConfig
+    from optimus.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3ParallelMoE
+    inp = sc.dsv3_inputs()
+    c = inp["cfg"]
+    rank = 2
+    blk = DeepseekV3ParallelMoE(DeepseekV3ParallelConfig(expert_parallelism=8),
+                                ParallelDpPpEpTpMapper(expert_parallelism=8, rank=rank)).to(device).to(torch.bfloat16)
+    with torch.no_grad():
+        blk.gate.weight.copy_(inp["router_w"]); blk.gate.e_score_correction_bias.copy_(inp["bias"])
+        for i, m in enumerate(blk.experts):
+            m.gate_proj.weight.copy_(inp["w_gate"][i]); m.up_proj.weight.copy_(inp["w_up"][i])
+            m.down_proj.weight.copy_(inp["w_down"][i])
+        blk.shared_experts.gate_proj.weight.copy_(inp["ws_gate"]); blk.shared_experts.up_proj.weight.copy_(inp["ws_up"])
+        blk.shared_experts.down_proj.weight.copy_(inp["ws_down"])
+    x = inp["x"].to(device).view(2, c["T"] // 2, c["H"]).requires_grad_(True)
+    dout = inp["dout"].to(device).view_as(x)
+    del inp
+
+    def step_c5():
+        for p in blk.parameters():
+            p.grad = None
+        x.grad = None
+        o = blk(x)
+        o.backward(dout)
+    ms, per = _timed_steps(step_c5, max(2, args.warmup // 2), steps)
+    with torch.no_grad():
+        e, _ = blk.gate(x.detach())
+        local = (e >= rank * c["NR"]) & (e < (rank + 1) * c["NR"])
+        tr = int(local.sum())
+        counts = torch.bincount((e[local] - rank * c["NR"]).flatten(), minlength=c["NR"])
+    flops = 18.0 * (tr + c["T"]) * c["H"] * c["I"]
+    wbytes = 3 * 3 * c["NR"] * c["H"] * c["I"] * 2
+    out["C5"] = entry(c["T"], ms, per, flops, wbytes, extra={
+        "workload": "C5 DeepSeek-V3-style layer, one GPU's share: 8192 tokens, hidden 7168, 32 local of 256 routed "
+                    "experts (ffn 2048) + 1 shared expert, sigmoid group-limited top-8 router; fwd+bwd",
+        "routed_rows_on_this_rank": tr,
+        "rows_per_expert": {"min": int(counts.min()), "median": int(counts.median()), "max": int(counts.max())},
+        "note": "expert_gemm_* and mfma_frac cover the routed and the shared expert's products together; "
+                "weight_stream_* counts the 32 routed experts' matrices only"})
+    del blk, x, dout
+    torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline_moe():
     """oracle.moe_layer.olmoe_slow_block (the reference's per-expert loop, fp32) forward+backward on
     1/16 of the C3 tokens with the full expert weights; tokens/s of that run."""
@@ -321,6 +488,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baselines")
     ap.add_argument("--skip-adamw", action="store_true", help="leave out the AdamW workload")
+    ap.add_argument("--skip-other", action="store_true", help="leave out the C1 / C4 / C5 configurations")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU's hot path; --gpus must be 1 "
@@ -345,6 +513,8 @@ def main():
     }
     # GPU workloads first, back to back: the seconds of CPU baseline in between would let the GPU
     # fall into its idle power state right before the HBM-bound measurement
+    if not args.skip_other:
+        out["other_configs"] = bench_other_configs(args, device, not args.skip_cpu)
     ad = None if args.skip_adamw else bench_adamw(args, device)
     if not args.skip_cpu:
         out["cpu_baseline"] = cpu_baseline_moe()

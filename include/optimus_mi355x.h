@@ -354,9 +354,10 @@ int om_rmsnorm_bwd(const void *dy, const void *h, const void *weight, const floa
  * w_stride: elements between the matrices of consecutive experts in `weight` /
  * `weight_grad`; 0 means densely packed (N*K, the merged [G,N,K] layout).  A larger stride
  * serves per-expert nn.Linear weights that sit at a constant pitch inside one flat buffer
- * (a multiple of 8 elements, else OM_ERR_ALIGN).  N and K must be multiples of 128.  Every
- * activation / weight tensor spans fewer than 2^35 elements (the kernels address operands in
- * 32-bit units of 16 bytes), e.g. 16M routed rows of 2048.  fwd and dgrad (and the merged-MLP fusions below) keep
+ * (a multiple of 8 elements, else OM_ERR_ALIGN).  N and K must be multiples of 128.  Tensors
+ * may exceed 2^31 elements (64-bit block-uniform bases, 32-bit offsets inside a tile); only a
+ * source whose rows are fetched through an index (the *_gathered / *_weighted forms below) must
+ * span fewer than 2^31 elements, e.g. 1M tokens of 2048.  fwd and dgrad (and the merged-MLP fusions below) keep
  * a per-expert tile table in LDS and take G <= 1024 (OM_ERR_SHAPE above that); wgrad has no
  * such limit.                                                                             */
 int om_grouped_gemm_fwd(const void *input, const void *weight, void *output,

@@ -99,6 +99,14 @@ __device__ __forceinline__ void load16_to_lds(const void *gptr, char *lds_base) 
     __builtin_amdgcn_global_load_lds((glb_void_ptr)gptr, (lds_void_ptr)lds_base, 16, 0, 0);
 }
 
+// A block-uniform 64-bit value, pinned to scalar registers (the compiler cannot always prove that
+// per-tile state carried around the tile loop is uniform).
+__device__ __forceinline__ int64_t uniform64(int64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(static_cast<uint64_t>(v) >> 32));
+    return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 // ---- CONTIG tile: R rows x 64 c; 128-byte rows; chunk position = chunk ^ swz(row) ----------
 // (row >> 1) & 7: measured conflict-free for ds_read_b128 with 32 consecutive rows per half-wave
 // (counter SQ_LDS_BANK_CONFLICT = 0, 4 cycles per read); period 16, so rows 32 apart share it.
@@ -307,6 +315,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);   // the same value in a scalar register
 
     // ---- per-tile state (set by setup_tile) ---------------------------------------------------
     int expert = 0, row_begin = 0, row_end = 0;  // fwd/dgrad: rows of this tile's expert segment
@@ -326,12 +335,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // ---- per-lane source offsets of the direct loads (elements, without the c0 term) ------------
     // CONTIG : lane -> (row = group*8 + lane/8, chunk = (lane%8) ^ swz(row))
     // STRIDED: lane -> (crow = group*(64/CPR) + lane/CPR, chunk = (lane%CPR) ^ ((crow&3)<<2))
-    // in units of 16 bytes (8 elements): every row pitch, expert pitch, tile origin and contraction
-    // step is a multiple of 8 elements, and the host checks that every operand spans < 2^32 units
-    uint32_t a_off[A_LOADS], b_off[B_LOADS];
+    // A load's address is (operand pointer + block-uniform 64-bit tile base) + a 32-bit per-lane
+    // offset: the wide part stays in scalar registers (the load takes a scalar base and a 32-bit
+    // vector offset), so operands of any size cost no vector arithmetic.  The per-lane part covers
+    // one tile (BM rows, or 64 contraction rows) — except for rows fetched through an index, whose
+    // lane offset is index * pitch: such a source must span < 2^31 elements (checked on the host).
+    int a_off[A_LOADS], b_off[B_LOADS];
+    int64_t a_base = 0, b_base = 0;   // elements, block-uniform
     int a_crow[A_LOADS];  // STRIDED A in wgrad: c-row of the lane's slot (for the zero fill)
     int b_crow[B_LOADS];
-    bool b_up[B_LOADS];   // EPI_SWIGLU: this LDS row comes from the up matrix
     int b_src[GATHER == GATHER_B ? B_LOADS : 1];   // GATHER_B: source rows of the next B loads
     int a_src[GATHER == GATHER_WA ? A_LOADS : 1];  // GATHER_WA: source rows of the next A loads
 #pragma unroll
@@ -344,10 +356,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         constexpr int CPR = BN / 8;
         const int grp = wave * B_LOADS + i;
         b_crow[i] = (BKIND == CONTIG) ? 0 : grp * (64 / CPR) + lane / CPR;
-        b_up[i] = (EPI == EPI_SWIGLU) ? (((grp * 8 + (lane >> 3)) >> 5) & 1) : false;
     }
 
-    const uint32_t lda16 = static_cast<uint32_t>(p.lda >> 3), ldb16 = static_cast<uint32_t>(p.ldb >> 3);
+    const int lda32 = static_cast<int>(p.lda), ldb32 = static_cast<int>(p.ldb);
     // GATHER_B: the B rows that contraction step `step` needs, looked up one step ahead of the
     // loads that use them (plain loads: they land before the next wait for the direct loads).
     auto index_of = [&](int step, int c0, int c) -> int {   // c0: the step's first row (block-uniform)
@@ -425,14 +436,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             if (AKIND == CONTIG) {
                 const int row = grp * 8 + (lane_s >> 3);
                 const int ch = (lane_s & 7) ^ swz(row);
-                int64_t m = static_cast<int64_t>(row_begin) + row;
+                int m = row_begin + row;
                 if (m >= row_end) m = row_end - 1;  // rows past the segment: valid memory, result unused
                 if (GATHER == GATHER_A) m = p.row_index[m];
-                a_off[i] = static_cast<uint32_t>(((m * p.lda) >> 3) + ch);
+                else m -= row_begin;                // the tile's first row is part of a_base
+                a_off[i] = m * lda32 + ch * 8;
             } else {
                 constexpr int CPR = BM / 8;
                 const int ch = (lane_s % CPR) ^ ((a_crow[i] & 3) << 2);
-                a_off[i] = static_cast<uint32_t>((row_begin >> 3) + ch);  // + (c_begin + c) * lda16 per step
+                a_off[i] = row_begin + ch * 8;  // + (contraction row within the step) * lda per step
             }
         }
 #pragma unroll
@@ -444,17 +456,24 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                 if (EPI == EPI_SWIGLU) {
                     // LDS rows alternate 32 gate rows / 32 up rows; the up matrix is B[1]
                     const int blk = row >> 5;
-                    const int64_t n = n0 + (blk >> 1) * 32 + (row & 31);
-                    b_off[i] = static_cast<uint32_t>(((expert * p.strideB + n * p.ldb) >> 3) + ch);
+                    const int n = (blk >> 1) * 32 + (row & 31);
+                    b_off[i] = n * ldb32 + ch * 8;
                 } else {
-                    b_off[i] = static_cast<uint32_t>(((expert * p.strideB + static_cast<int64_t>(n0 + row) * p.ldb) >> 3) + ch);
+                    b_off[i] = row * ldb32 + ch * 8;
                 }
             } else {
                 constexpr int CPR = BN / 8;
                 const int ch = (lane_s % CPR) ^ ((b_crow[i] & 3) << 2);
-                b_off[i] = static_cast<uint32_t>((((EPI == EPI_WGRAD ? 0 : expert * p.strideB) + n0) >> 3) + ch);
+                // fwd/dgrad: the lane's contraction row within a step never changes, so it is part of
+                // the offset; wgrad clamps the row into the expert's segment per step
+                b_off[i] = ch * 8 + (EPI == EPI_WGRAD ? 0 : b_crow[i] * ldb32);
             }
         }
+        // block-uniform parts of the addresses (scalar registers)
+        if (AKIND == CONTIG) a_base = GATHER == GATHER_A ? 0 : static_cast<int64_t>(row_begin) * p.lda;
+        else a_base = 0;   // wgrad: the contraction rows enter per step (step_base)
+        if (BKIND == CONTIG) b_base = expert * p.strideB + static_cast<int64_t>(n0) * p.ldb;
+        else b_base = (EPI == EPI_WGRAD ? 0 : expert * p.strideB) + n0;
         if (GATHER_W && expert != cached_expert) {
             // every wavefront is past the barrier that ends the previous tile's main loop, so no
             // one still reads the cache; `expert` is block-uniform, so all take this branch together
@@ -478,27 +497,32 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         const int sp = step - ph * steps_per_phase;
         int c0 = (sp < steps_per_phase ? rotated(sp) : sp) * BK;   // padding steps stay past the end
         if (EPI != EPI_WGRAD && c0 > c_len - BK) c0 = c_len - BK;
-        const char *Ap = reinterpret_cast<const char *>(p.phases > 1 && ph ? p.A[1] : p.A[0]);
+        // first contraction row that this step's STRIDED loads may touch, folded into the scalar base
+        // (rows are clamped into the segment, so the base is clamped the same way)
+        const int c_lo = (EPI == EPI_WGRAD) ? max(min(c0, c_len - 1), 0) : c0;
+        const int64_t a_step = uniform64(a_base + ((AKIND == STRIDED && GATHER != GATHER_WA) ? static_cast<int64_t>(c_begin + c_lo) * p.lda : 0));
+        const int64_t b_step = uniform64(b_base + ((BKIND == STRIDED && GATHER != GATHER_B) ? static_cast<int64_t>(c_begin + c_lo) * p.ldb : 0));
+        const char *Ap = reinterpret_cast<const char *>((p.phases > 1 && ph ? p.A[1] : p.A[0]) + a_step);
         const char *Bp = reinterpret_cast<const char *>(
-            (EPI != EPI_SWIGLU && p.phases > 1 && ph) ? p.B[1] : p.B[0]);
-        const char *Bup = reinterpret_cast<const char *>(p.B[1]);
+            ((EPI != EPI_SWIGLU && p.phases > 1 && ph) ? p.B[1] : p.B[0]) + b_step);
+        const char *Bup = reinterpret_cast<const char *>(p.B[1] + b_step);
         char *sa = stage + wave * (A_LOADS * 1024);
         char *sb = stage + A_BYTES + wave * (B_LOADS * 1024);
 #pragma unroll
         for (int i = 0; i < A_LOADS; i++) {
             if (i < lo || i >= hi) continue;
-            uint32_t off;  // 16-byte units from the operand base; < 2^32 (checked on the host)
+            uint32_t off;  // bytes from the step's scalar base
             if (AKIND == CONTIG) {
-                off = a_off[i] + static_cast<uint32_t>(c0 >> 3);
+                off = static_cast<uint32_t>(a_off[i] + c0) * 2u;
             } else {
                 int c = c0 + a_crow[i];
                 if (EPI == EPI_WGRAD) c = min(c, c_len - 1);  // stay in the segment; zeroed below
                 if (GATHER == GATHER_WA)
-                    off = a_off[i] + static_cast<uint32_t>(a_src[GATHER == GATHER_WA ? i : 0]) * lda16;
+                    off = static_cast<uint32_t>(a_off[i] + a_src[GATHER == GATHER_WA ? i : 0] * lda32) * 2u;
                 else
-                    off = a_off[i] + static_cast<uint32_t>(c_begin + c) * lda16;
+                    off = static_cast<uint32_t>(a_off[i] + (c - c_lo) * lda32) * 2u;
             }
-            load16_to_lds(Ap + (static_cast<uint64_t>(off) << 4), sa + i * 1024);
+            load16_to_lds(Ap + off, sa + i * 1024);
         }
         if (hi >= A_LOADS && lo < A_LOADS) load_a_src(step + 1);   // this step's A loads are out
 #pragma unroll
@@ -506,16 +530,25 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             if (A_LOADS + i < lo || A_LOADS + i >= hi) continue;
             uint32_t off;
             if (BKIND == CONTIG) {
-                off = b_off[i] + static_cast<uint32_t>(c0 >> 3);
+                off = static_cast<uint32_t>(b_off[i] + c0) * 2u;
             } else {
-                int c = c0 + b_crow[i];
-                if (EPI == EPI_WGRAD) c = min(c, c_len - 1);
-                if (GATHER == GATHER_B)
-                    off = b_off[i] + static_cast<uint32_t>(b_src[GATHER == GATHER_B ? i : 0]) * ldb16;
-                else
-                    off = b_off[i] + static_cast<uint32_t>(c_begin + c) * ldb16;
+                if (GATHER == GATHER_B) {
+                    off = static_cast<uint32_t>(b_off[i] + b_src[GATHER == GATHER_B ? i : 0] * ldb32) * 2u;
+                } else if (EPI == EPI_WGRAD) {
+                    const int c = min(c0 + b_crow[i], c_len - 1);
+                    off = static_cast<uint32_t>(b_off[i] + (c - c_lo) * ldb32) * 2u;
+                } else {
+                    // loop-invariant: kept opaque so that it stays a 32-bit register next to a scalar
+                    // base (hoisted, it becomes a zero-extended 64-bit pair per load)
+                    int o = b_off[i];
+                    asm volatile("" : "+v"(o));
+                    off = static_cast<uint32_t>(o) * 2u;
+                }
             }
-            load16_to_lds(((EPI == EPI_SWIGLU && b_up[i]) ? Bup : Bp) + (static_cast<uint64_t>(off) << 4), sb + i * 1024);
+            // EPI_SWIGLU: a load covers 8 LDS rows inside one 32-row block, all gate or all up rows, so
+            // the choice of the matrix is uniform over the wavefront (scalar base, 32-bit lane offset)
+            const bool up_rows = EPI == EPI_SWIGLU && ((((wave_u * B_LOADS + i) * 8) >> 5) & 1);
+            load16_to_lds((up_rows ? Bup : Bp) + off, sb + i * 1024);
         }
         if (hi >= A_LOADS + B_LOADS && lo < A_LOADS + B_LOADS) load_b_src(step + 1);   // this step's B loads are out
     };
@@ -900,9 +933,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 // of 64x64) when an extent is not a multiple of 256 or experts hold few rows each.
 
 inline bool mult(int64_t v, int m) { return v > 0 && v % m == 0; }
-// the kernels address an operand in 32-bit units of 16 bytes: fewer than 2^35 elements per tensor,
-// and per-expert pitches that are multiples of 8 elements (16-byte vectors need that anyway)
-inline bool fits_span(int64_t elems) { return elems >= 0 && elems < (1LL << 35); }
+// Operands are addressed as a 64-bit block-uniform base plus a 32-bit lane offset, so their size is
+// only bounded by int64 arithmetic on element counts (2^40 here, far beyond device memory); a source
+// whose rows are fetched through an index has index * pitch in the lane offset and must span
+// < 2^31 elements.  Per-expert pitches are multiples of 8 elements (16-byte vectors need that).
+inline bool fits_span(int64_t elems) { return elems >= 0 && elems < (1LL << 40); }
+inline bool fits_gather(int64_t elems) { return elems >= 0 && elems < (1LL << 31); }
 inline bool pitch_ok(int64_t stride) { return stride >= 0 && stride % 8 == 0; }
 
 // Blocks of a launch: one resident set (a multiple of the 8 XCDs), or fewer when there are few
@@ -1027,7 +1063,7 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inde
     p.strideC = w_stride ? w_stride : static_cast<int64_t>(N) * K;
     if (!pitch_ok(p.strideC)) return OM_ERR_ALIGN;
     if (!fits_span(rows * K) || !fits_span(rows * N) || !fits_span(p.strideC * G) ||
-        !fits_span(src_rows * (gather == GATHER_WA ? N : K)))
+        !fits_gather(src_rows * (gather == GATHER_WA ? N : K)))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
     hipStream_t st = om_stream(stream);
@@ -1108,7 +1144,7 @@ int gate_up_fwd_launch(const void *x, const int32_t *x_rows, int64_t src_rows, c
     p.lda = H; p.ldb = H; p.ldc = I;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(I) * H;
     if (!pitch_ok(p.strideB)) return OM_ERR_ALIGN;
-    if (!fits_span(rows * H) || !fits_span(rows * I) || !fits_span(p.strideB * G) || !fits_span(src_rows * H))
+    if (!fits_span(rows * H) || !fits_span(rows * I) || !fits_span(p.strideB * G) || !fits_gather(src_rows * H))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = I; p.kc = H; p.phases = 1;
     if (row_weights) return launch_rows_auto<CONTIG, CONTIG, EPI_SWIGLU, GATHER_A, true>(p, rows, om_stream(stream));
@@ -1179,7 +1215,7 @@ int down_dgrad_launch(const void *dy, const int32_t *dy_rows, int64_t src_rows, 
     p.lda = H; p.ldb = I; p.ldc = I;
     p.strideB = w_stride ? w_stride : static_cast<int64_t>(H) * I;
     if (!pitch_ok(p.strideB)) return OM_ERR_ALIGN;
-    if (!fits_span(rows * H) || !fits_span(rows * I) || !fits_span(p.strideB * G) || !fits_span(src_rows * H))
+    if (!fits_span(rows * H) || !fits_span(rows * I) || !fits_span(p.strideB * G) || !fits_gather(src_rows * H))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = I; p.kc = H; p.phases = 1;
     if (dy_rows) return launch_rows_auto<CONTIG, STRIDED, EPI_SWIGLU_BWD, GATHER_A, true>(p, rows, om_stream(stream));

@@ -139,7 +139,7 @@ def test_grouped_gemms(lib):
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 4096, 1025, 256, 256, 0, None) == SHAPE      # G > 1024 (LDS table)
     assert lib.om_grouped_gemm_fwd(P, None, P, P, *args) == NULL
     assert lib.om_grouped_gemm_fwd(P, P, ODD, P, *args) == ALIGN
-    assert lib.om_grouped_gemm_fwd(P, P, P, P, 1 << 25, 64, 2048, 1024, 0, None) == SHAPE   # 2^35 elements or more
+    assert lib.om_grouped_gemm_fwd(P, P, P, P, 1 << 30, 64, 2048, 1024, 0, None) == SHAPE   # 2^40 elements or more
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 4096, 64, 2048, 1024, 2048 * 1024 + 4, None) == ALIGN   # expert pitch % 8
     assert lib.om_grouped_gemm_dgrad(P, P, P, None, *args) == NULL
     assert lib.om_grouped_gemm_wgrad(P, P, P, P, 131072, 0, 2048, 1024, 0, None) == SHAPE   # G < 1
@@ -159,7 +159,7 @@ def test_grouped_gemms(lib):
     g = (131072, 64, 1024, 2048, 0, None)
     assert lib.om_merged_mlp_gate_up_fwd_gathered(P, None, 16384, P, P, P, P, P, P, *g) == NULL      # no index
     assert lib.om_merged_mlp_gate_up_fwd_gathered(P, P, 0, P, P, P, P, P, P, *g) == SHAPE            # no source rows
-    assert lib.om_merged_mlp_gate_up_fwd_gathered(P, P, 1 << 24, P, P, P, P, P, P, *g) == SHAPE      # source of 2^35 elements or more
+    assert lib.om_merged_mlp_gate_up_fwd_gathered(P, P, 1 << 20, P, P, P, P, P, P, *g) == SHAPE      # indexed source of 2^31 elements or more
     assert lib.om_merged_mlp_gate_up_fwd_gathered(P, None, 0, P, P, P, P, P, P, 0, 64, 1024, 2048, 0, None) == OK
     assert lib.om_grouped_gemm_wgrad_gathered(P, P, None, 16384, P, P, *g) == NULL
     assert lib.om_grouped_gemm_wgrad_gathered(P, P, P, 0, P, P, *g) == SHAPE
@@ -183,7 +183,7 @@ def test_routing_weight_folded_into_the_expert_mlp(lib):
     gw = (131072, 64, 2048, 1024, 0, None)
     assert lib.om_grouped_gemm_wgrad_gathered_out(P, None, 16384, P, P, P, *gw) == NULL
     assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 0, P, P, P, *gw) == SHAPE
-    assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 1 << 25, P, P, P, *gw) == SHAPE   # source of 2^35 elements or more
+    assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 1 << 21, P, P, P, *gw) == SHAPE   # indexed source of 2^31 elements or more
     assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 16384, P, ODD, P, *gw) == ALIGN
     assert lib.om_merged_mlp_row_dot_parts(1024) == 16
     assert lib.om_merged_mlp_row_dot_parts(100) == SHAPE
