@@ -50,7 +50,11 @@ def _ref_fwd(x, w, cum):
     return out
 
 
-CASES = [("uniform", 4, 512, 256, 128), ("ragged", 8, 1000, 256, 512), ("empties", 16, 777, 128, 256),
+CASES = [# few rows per expert with extents that are multiples of 256 (skewed small batches): most tiles hold
+         # a handful of valid rows; one expert with many row tiles among empty ones
+         ("ragged", 64, 4096, 1024, 2048), ("empties", 64, 3000, 256, 512), ("onehot", 16, 1000, 256, 256),
+         ("uniform", 20, 640, 512, 256), ("ragged", 300, 9000, 256, 256), ("ragged", 512, 4097, 256, 512),
+         ("uniform", 4, 512, 256, 128), ("ragged", 8, 1000, 256, 512), ("empties", 16, 777, 128, 256),
          ("ragged", 64, 4096, 1024, 2048), ("uniform", 1, 300, 256, 256), ("ragged", 3, 5, 128, 128),
          # several tiles per persistent block, on both tile shapes, with empty experts in between
          ("ragged", 8, 20000, 512, 768), ("ragged", 8, 20000, 384, 640), ("empties", 32, 9000, 512, 1024),
@@ -94,6 +98,9 @@ def test_grouped_gemm_fwd_dgrad_wgrad(cuda, kind, G, rows, N, K):
 
 
 @pytest.mark.parametrize("kind,G,rows,I,H", [("uniform", 4, 512, 128, 256), ("ragged", 8, 1500, 512, 256),
+                                            # skewed small batches: a few rows per expert
+                                            ("ragged", 64, 4096, 1024, 2048), ("empties", 32, 700, 256, 512),
+                                            ("onehot", 8, 500, 128, 256), ("ragged", 40, 1000, 384, 256),
                                             ("empties", 64, 4096, 1024, 2048), ("ragged", 2, 7, 128, 128)])
 def test_merged_mlp_fused(cuda, kind, G, rows, I, H):
     """MergedMLP (fused gate+up+SwiGLU, fused down-dgrad+SwiGLU-backward, dual dgrad) against the

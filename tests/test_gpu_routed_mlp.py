@@ -91,6 +91,8 @@ NAMES = ("out", "dx", "d_routing_weights", "dw_gate", "dw_up", "dw_down", "d_res
     (512, 2, 8, 0, 8, 128, 384, 0.0, torch.bfloat16),       # 128x128 tiles, bf16 routing weights
     (1500, 4, 16, 4, 12, 256, 256, 1.5, torch.float32),     # expert window: some pairs are not routed
     (70, 8, 64, 0, 64, 128, 128, 3.0, torch.float32),       # most experts empty, a few rows each
+    (512, 8, 64, 0, 64, 1024, 2048, 1.2, torch.bfloat16),   # the skewed small batch: a few rows per expert
+    (300, 4, 32, 8, 24, 256, 512, 2.0, torch.float32),      # the same with an expert window
 ])
 @pytest.mark.parametrize("residual", [False, True])
 def test_routed_mlp_against_float32_and_separate_functions(cuda, T, K, N, start, end, I, H, skew, wdt, residual):
