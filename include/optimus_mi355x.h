@@ -194,6 +194,19 @@ int om_router_gate_dgrad(const float *dlogits, const void *gate_weight, const vo
  * om_router_balance_bwd: dlogits[t,i] = p_i * (g_i - sum_j p_j g_j) with g = prob_grad [N] fp32,
  *   the gradient of the loss with respect to prob_sum (the counts carry no gradient).      */
 int64_t om_router_balance_workspace_bytes(int64_t T, int N);
+/* The *_masked forms take the attention mask of the same function
+ * (optimus/models/olmoe/modeling_olmoe.py:58-83) as one weight per token, token_weight [T] fp32
+ * (the mask entry of the token's batch row and position; null = every token counts once):
+ *   prob_sum[e] = sum_t token_weight[t] * softmax(logits[t,:])[e]
+ *   count[e]    = sum_t token_weight[t] * [e in top-K of token t]
+ * and dlogits[t,i] = token_weight[t] * p_i * (g_i - sum_j p_j g_j) backward.  The caller divides by
+ * the sum of the weights (all layers share one mask).                                          */
+int om_router_balance_stats_masked(const void *logits, int logits_dtype, const float *token_weight,
+                                   int64_t T, int N, int K, float *prob_sum, float *count,
+                                   void *workspace, int64_t workspace_bytes, void *stream);
+int om_router_balance_bwd_masked(const void *logits, int logits_dtype, const float *prob_grad,
+                                 const float *token_weight, int64_t T, int N, void *dlogits,
+                                 void *stream);
 int om_router_balance_stats(const void *logits, int logits_dtype, int64_t T, int N, int K,
                             float *prob_sum, float *count, void *workspace,
                             int64_t workspace_bytes, void *stream);

@@ -399,32 +399,34 @@ int launch_gate(const void *x, const void *wg, int64_t T, int H, int N, int K, i
 // kernel adds the rows in block order, so the result does not depend on scheduling.
 constexpr int BAL_TOKENS = 64;
 template <int PER, typename T>
-__global__ __launch_bounds__(256) void balance_stats_kernel(const T *__restrict__ logits, int64_t Tn,
-                                                            int N, int K,
+__global__ __launch_bounds__(256) void balance_stats_kernel(const T *__restrict__ logits,
+                                                            const float *__restrict__ token_weight,
+                                                            int64_t Tn, int N, int K,
                                                             float *__restrict__ part_prob,
-                                                            int *__restrict__ part_count) {
+                                                            float *__restrict__ part_count) {
     __shared__ float lds_p[4][PER * 64];
-    __shared__ int lds_c[4][PER * 64];
+    __shared__ float lds_c[4][PER * 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float psum[PER];
-    int cnt[PER];
+    float cnt[PER];   // sums of token weights; whole numbers (exact) for 0/1 weights and without weights
 #pragma unroll
-    for (int j = 0; j < PER; j++) { psum[j] = 0.0f; cnt[j] = 0; }
+    for (int j = 0; j < PER; j++) { psum[j] = 0.0f; cnt[j] = 0.0f; }
     const int64_t t_first = static_cast<int64_t>(blockIdx.x) * BAL_TOKENS;
     for (int i = wave; i < BAL_TOKENS; i += 4) {
         const int64_t t = t_first + i;
         if (t >= Tn) break;
+        const float tw = token_weight ? token_weight[t] : 1.0f;   // the token's attention-mask entry
         float p[PER], s[PER];
         row_softmax<PER, T>(logits + t * N, N, lane, p);
 #pragma unroll
-        for (int j = 0; j < PER; j++) { psum[j] += p[j]; s[j] = p[j]; }
+        for (int j = 0; j < PER; j++) { psum[j] += token_weight ? tw * p[j] : p[j]; s[j] = p[j]; }
         float w; int e;
         select_topk<PER>(s, N, K, lane, w, e);
         for (int k = 0; k < K; k++) {
             const int ek = __shfl(e, k, 64);
 #pragma unroll
             for (int j = 0; j < PER; j++)
-                if (lane + 64 * j == ek) cnt[j]++;
+                if (lane + 64 * j == ek) cnt[j] += tw;
         }
     }
 #pragma unroll
@@ -432,32 +434,32 @@ __global__ __launch_bounds__(256) void balance_stats_kernel(const T *__restrict_
     __syncthreads();
     for (int i = threadIdx.x; i < N; i += 256) {
         part_prob[static_cast<int64_t>(blockIdx.x) * N + i] = (lds_p[0][i] + lds_p[1][i]) + (lds_p[2][i] + lds_p[3][i]);
-        part_count[static_cast<int64_t>(blockIdx.x) * N + i] = lds_c[0][i] + lds_c[1][i] + lds_c[2][i] + lds_c[3][i];
+        part_count[static_cast<int64_t>(blockIdx.x) * N + i] = (lds_c[0][i] + lds_c[1][i]) + (lds_c[2][i] + lds_c[3][i]);
     }
 }
 
 __global__ __launch_bounds__(256) void balance_reduce_kernel(const float *__restrict__ part_prob,
-                                                             const int *__restrict__ part_count,
+                                                             const float *__restrict__ part_count,
                                                              int n_blocks, int N,
                                                              float *__restrict__ prob_sum,
                                                              float *__restrict__ count) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= N) return;
-    float ps = 0.0f;
-    int c = 0;
+    float ps = 0.0f, c = 0.0f;
     for (int b = 0; b < n_blocks; b++) {
         ps += part_prob[static_cast<int64_t>(b) * N + i];
-        c += part_count[static_cast<int64_t>(b) * N + i];
+        c += part_count[static_cast<int64_t>(b) * N + i];   // whole numbers below 2^24: exact
     }
     prob_sum[i] = ps;
-    count[i] = static_cast<float>(c);
+    count[i] = c;
 }
 
 // dlogits[t,i] = p_i * (g_i - sum_j p_j g_j): the softmax backward of sum_i g_i * p[t,i].
 template <int PER, typename T>
 __global__ __launch_bounds__(256) void balance_bwd_kernel(const T *__restrict__ logits,
-                                                          const float *__restrict__ g, int64_t Tn,
-                                                          int N, T *__restrict__ dlogits) {
+                                                          const float *__restrict__ g,
+                                                          const float *__restrict__ token_weight,
+                                                          int64_t Tn, int N, T *__restrict__ dlogits) {
     const int lane = threadIdx.x & 63;
     const int64_t t = static_cast<int64_t>(blockIdx.x) * TOKENS_PER_BLOCK + (threadIdx.x >> 6);
     if (t >= Tn) return;
@@ -474,7 +476,7 @@ __global__ __launch_bounds__(256) void balance_bwd_kernel(const T *__restrict__ 
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         const int i = lane + 64 * j;
-        if (i < N) Elem<T>::store(dlogits + t * N + i, p[j] * (gv[j] - dot));
+        if (i < N) Elem<T>::store(dlogits + t * N + i, (token_weight ? token_weight[t] : 1.0f) * (p[j] * (gv[j] - dot)));
     }
 }
 
@@ -608,9 +610,10 @@ extern "C" int64_t om_router_balance_workspace_bytes(int64_t T, int N) {
     return blocks * N * 8;   // one float and one int per (block, expert)
 }
 
-extern "C" int om_router_balance_stats(const void *logits, int logits_dtype, int64_t T, int N, int K,
-                                       float *prob_sum, float *count, void *workspace,
-                                       int64_t workspace_bytes, void *stream) {
+extern "C" int om_router_balance_stats_masked(const void *logits, int logits_dtype,
+                                              const float *token_weight, int64_t T, int N, int K,
+                                              float *prob_sum, float *count, void *workspace,
+                                              int64_t workspace_bytes, void *stream) {
     if (logits_dtype != OM_F32 && logits_dtype != OM_BF16) return OM_ERR_DTYPE;
     if (T < 1 || N < 1 || N > 512 || K < 1 || K > N || K > 64 || T > 0x7fffffffLL) return OM_ERR_SHAPE;
     if (!logits || !prob_sum || !count || !workspace) return OM_ERR_NULL;
@@ -618,20 +621,28 @@ extern "C" int om_router_balance_stats(const void *logits, int logits_dtype, int
     hipStream_t st = om_stream(stream);
     const int nb = static_cast<int>((T + BAL_TOKENS - 1) / BAL_TOKENS);
     float *pp = static_cast<float *>(workspace);
-    int *pc = reinterpret_cast<int *>(pp + static_cast<int64_t>(nb) * N);
+    float *pc = pp + static_cast<int64_t>(nb) * N;
     if (logits_dtype == OM_F32) {
         OM_DISPATCH_PER(N, (balance_stats_kernel<PER, float><<<nb, 256, 0, st>>>(
-                               static_cast<const float *>(logits), T, N, K, pp, pc)));
+                               static_cast<const float *>(logits), token_weight, T, N, K, pp, pc)));
     } else {
         OM_DISPATCH_PER(N, (balance_stats_kernel<PER, uint16_t><<<nb, 256, 0, st>>>(
-                               static_cast<const uint16_t *>(logits), T, N, K, pp, pc)));
+                               static_cast<const uint16_t *>(logits), token_weight, T, N, K, pp, pc)));
     }
     balance_reduce_kernel<<<(N + 255) / 256, 256, 0, st>>>(pp, pc, nb, N, prob_sum, count);
     return om_launch_status();
 }
 
-extern "C" int om_router_balance_bwd(const void *logits, int logits_dtype, const float *prob_grad,
-                                     int64_t T, int N, void *dlogits, void *stream) {
+extern "C" int om_router_balance_stats(const void *logits, int logits_dtype, int64_t T, int N, int K,
+                                       float *prob_sum, float *count, void *workspace,
+                                       int64_t workspace_bytes, void *stream) {
+    return om_router_balance_stats_masked(logits, logits_dtype, nullptr, T, N, K, prob_sum, count,
+                                          workspace, workspace_bytes, stream);
+}
+
+extern "C" int om_router_balance_bwd_masked(const void *logits, int logits_dtype, const float *prob_grad,
+                                            const float *token_weight, int64_t T, int N, void *dlogits,
+                                            void *stream) {
     if (logits_dtype != OM_F32 && logits_dtype != OM_BF16) return OM_ERR_DTYPE;
     if (T < 0 || N < 1 || N > 512 || T > 0x7fffffffLL) return OM_ERR_SHAPE;
     if (T == 0) return OM_OK;
@@ -640,12 +651,17 @@ extern "C" int om_router_balance_bwd(const void *logits, int logits_dtype, const
     const unsigned nb = token_blocks(T);
     if (logits_dtype == OM_F32) {
         OM_DISPATCH_PER(N, (balance_bwd_kernel<PER, float><<<nb, 256, 0, st>>>(
-                               static_cast<const float *>(logits), prob_grad, T, N,
+                               static_cast<const float *>(logits), prob_grad, token_weight, T, N,
                                static_cast<float *>(dlogits))));
     } else {
         OM_DISPATCH_PER(N, (balance_bwd_kernel<PER, uint16_t><<<nb, 256, 0, st>>>(
-                               static_cast<const uint16_t *>(logits), prob_grad, T, N,
+                               static_cast<const uint16_t *>(logits), prob_grad, token_weight, T, N,
                                static_cast<uint16_t *>(dlogits))));
     }
     return om_launch_status();
+}
+
+extern "C" int om_router_balance_bwd(const void *logits, int logits_dtype, const float *prob_grad,
+                                     int64_t T, int N, void *dlogits, void *stream) {
+    return om_router_balance_bwd_masked(logits, logits_dtype, prob_grad, nullptr, T, N, dlogits, stream);
 }

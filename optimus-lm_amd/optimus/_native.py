@@ -52,6 +52,9 @@ SIGNATURES = {
     "om_router_balance_workspace_bytes": (c_i64, [c_i64, c_int]),
     "om_router_balance_stats": (c_int, [c_void_p, c_int, c_i64, c_int, c_int, c_void_p, c_void_p,
                                         c_void_p, c_i64, c_void_p]),
+    "om_router_balance_stats_masked": (c_int, [c_void_p, c_int, c_void_p, c_i64, c_int, c_int, c_void_p, c_void_p,
+                                               c_void_p, c_i64, c_void_p]),
+    "om_router_balance_bwd_masked": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_i64, c_int, c_void_p, c_void_p]),
     "om_router_balance_bwd": (c_int, [c_void_p, c_int, c_void_p, c_i64, c_int, c_void_p, c_void_p]),
     "om_rmsnorm_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_double, c_void_p, c_void_p, c_void_p,
                                c_i64, c_i64, c_int, c_void_p]),

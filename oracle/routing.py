@@ -90,16 +90,31 @@ def dsv3_router(hidden_states, weight, bias, n_group, topk_group, top_k, norm_to
     return topk_indices, topk_weights, router_logits
 
 
-def load_balancing_loss(gate_logits, num_experts, top_k):
-    """The reference's global auxiliary loss without a mask, optimus/models/olmoe/modeling_olmoe.py:
-    39-46 and :84-85, as the torch expressions it uses (softmax, topk, one_hot, two means), in the
-    dtype of the logits.  `gate_logits` is a tuple of per-layer [T,N] tensors."""
+def load_balancing_loss(gate_logits, num_experts, top_k, attention_mask=None):
+    """The reference's global auxiliary loss, optimus/models/olmoe/modeling_olmoe.py:39-85, as the
+    torch expressions it uses (softmax, topk, one_hot, means or masked sums), in the dtype of the
+    logits.  `gate_logits` is a tuple of per-layer [T,N] tensors; `attention_mask` [batch, sequence]
+    with batch * sequence == T selects the masked branch (:58-83)."""
     cat = torch.cat(list(gate_logits), dim=0)                                        # :41
     routing_weights = torch.nn.functional.softmax(cat, dim=-1)                       # :43
     _, selected = torch.topk(routing_weights, top_k, dim=-1)                         # :45
     expert_mask = torch.nn.functional.one_hot(selected, num_experts)                 # :47
-    tokens_per_expert = torch.mean(expert_mask.float(), dim=0)                       # :51
-    router_prob_per_expert = torch.mean(routing_weights, dim=0)                      # :54
+    if attention_mask is None:
+        tokens_per_expert = torch.mean(expert_mask.float(), dim=0)                   # :51
+        router_prob_per_expert = torch.mean(routing_weights, dim=0)                  # :54
+    else:
+        batch_size, sequence_length = attention_mask.shape                           # :56
+        num_hidden_layers = cat.shape[0] // (batch_size * sequence_length)           # :57
+        expert_attention_mask = (attention_mask[None, :, :, None, None]
+                                 .expand((num_hidden_layers, batch_size, sequence_length, top_k, num_experts))
+                                 .reshape(-1, top_k, num_experts))                   # :60-65
+        tokens_per_expert = torch.sum(expert_mask.float() * expert_attention_mask, dim=0) / torch.sum(
+            expert_attention_mask, dim=0)                                            # :68-70
+        router_mask = (attention_mask[None, :, :, None]
+                       .expand((num_hidden_layers, batch_size, sequence_length, num_experts))
+                       .reshape(-1, num_experts))                                    # :73-78
+        router_prob_per_expert = torch.sum(routing_weights * router_mask, dim=0) / torch.sum(
+            router_mask, dim=0)                                                      # :81-83
     return torch.sum(tokens_per_expert * router_prob_per_expert.unsqueeze(0)) * num_experts   # :84-85
 
 

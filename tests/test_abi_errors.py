@@ -86,6 +86,11 @@ def test_routers(lib):
     assert lib.om_grad_scale(ODD, 100, BF16, P, None) == ALIGN
     assert lib.om_grad_scale(None, 0, BF16, None, None) == OK
     assert lib.om_adamw_traffic_probe(P, P, P, None, P, 1024, None) == NULL
+    assert lib.om_router_balance_stats_masked(P, 7, P, 100, 64, 8, P, P, P, 1 << 20, None) == DTYPE
+    assert lib.om_router_balance_stats_masked(P, F32, None, 100, 64, 65, P, P, P, 1 << 20, None) == SHAPE
+    assert lib.om_router_balance_stats_masked(P, F32, P, 100, 64, 8, P, P, P, 8, None) == WORKSPACE
+    assert lib.om_router_balance_bwd_masked(P, F32, None, P, 100, 64, P, None) == NULL
+    assert lib.om_router_balance_bwd_masked(None, F32, None, None, 0, 64, None, None) == OK
     assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 64, None, BF16, P, need, None) == NULL
     assert lib.om_router_gate_wgrad(P, None, 16384, 2048, 64, P, BF16, P, need, None) == NULL
     assert lib.om_router_gate_wgrad(P, P, 16384, 2048, 64, ODD, BF16, P, need, None) == ALIGN

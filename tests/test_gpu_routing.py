@@ -372,3 +372,43 @@ def test_gate_shapes_without_a_kernel_raise(cuda):
                        torch.zeros(16, 8, device=cuda), (False, True))                      # weight gradient: H % 128
     with pytest.raises(TypeError):
         fp32_logits(x, torch.zeros(8, 192, dtype=torch.float32, device=cuda))              # mixed dtypes
+
+
+@pytest.mark.parametrize("L,B,S,N,K,dtype", [(3, 4, 1024, 64, 8, torch.float32), (2, 5, 200, 100, 5, torch.float32),
+                                             (1, 1, 77, 256, 8, torch.float32), (2, 2, 48, 16, 2, torch.bfloat16),
+                                             (4, 2, 256, 8, 2, torch.float32)])
+def test_masked_balance_loss_matches_the_reference_expression(cuda, L, B, S, N, K, dtype):
+    """load_balancing_loss_func with an attention mask (modeling_olmoe.py:58-83): value against the
+    oracle's restatement of the masked branch, gradient against autograd through it; masked tokens get
+    exactly zero gradient; an all-ones mask gives the unmasked loss."""
+    from optimus.models.common.ral_functions import load_balancing_loss_func
+    T = B * S
+    def layer_logits(seed):
+        if dtype == torch.float32:
+            return _valid_logits(T, N, K, seed=seed)
+        while True:    # the ROUNDED logits must order every token's top-(K+1) without ties
+            lg = (torch.randn(T, N, generator=torch.Generator().manual_seed(seed)) * 4.0).to(dtype).float()
+            if R.min_topk_gap_ulps(torch.softmax(lg, 1), K) > 4.0:
+                return lg
+            seed += 1000
+    layers = tuple(layer_logits(17 * l + T + N) for l in range(L))
+    g = torch.Generator().manual_seed(L + N)
+    mask = (torch.rand(B, S, generator=g) > 0.3).long()
+    mask[0, 0] = 1
+    dev = tuple(l.to(dtype).to(cuda).requires_grad_(True) for l in layers)
+    got = load_balancing_loss_func(dev, N, K, attention_mask=mask.to(cuda))
+    got.backward()
+    ref_in = tuple(l.to(dtype).float().requires_grad_(True) for l in layers)
+    want = R.load_balancing_loss(ref_in, N, K, attention_mask=mask.float())
+    want.backward()
+    tol = 2e-5 if dtype == torch.float32 else 2e-3
+    assert abs(float(got.detach()) - float(want.detach())) <= tol * float(want.detach())
+    keep = mask.reshape(-1).bool()
+    for a, b in zip(dev, ref_in):
+        ga = a.grad.float().cpu()
+        assert float(ga[~keep].abs().max()) == 0.0 if bool((~keep).any()) else True
+        err = float((ga - b.grad).abs().max())
+        assert err <= (1e-3 if dtype == torch.float32 else 2e-2) * float(b.grad.abs().max()) + 1e-12, err
+    ones = load_balancing_loss_func(tuple(d.detach() for d in dev), N, K, attention_mask=torch.ones(B, S, device=cuda))
+    plain = load_balancing_loss_func(tuple(d.detach() for d in dev), N, K)
+    assert abs(float(ones) - float(plain)) <= 1e-6 * float(plain)

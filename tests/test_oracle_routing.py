@@ -129,3 +129,31 @@ def test_balance_loss_closed_forms():
         logits[t, t % N] = 1.0; logits[t, (t + 1) % N] = 0.5
     loss = float(R.load_balancing_loss((logits,), N, K))
     assert abs(loss - K) < 1e-3
+
+
+def test_masked_balance_loss_is_the_loss_of_the_kept_tokens():
+    """Pins the masked branch of the auxiliary-loss restatement (modeling_olmoe.py:58-83) without
+    retyping it: with a 0/1 mask the loss must equal the unmasked loss evaluated on the kept tokens
+    alone (every layer's rows filtered by the same mask); an all-ones mask changes nothing; and the
+    plausible mistakes — dividing by the token count instead of the mask sum, or masking only one
+    of the two factors — give a different value."""
+    g = torch.Generator().manual_seed(4)
+    B, S, N, K, L = 3, 40, 16, 4, 3
+    layers = tuple(torch.randn(B * S, N, generator=g) * 2 for _ in range(L))
+    mask = (torch.rand(B, S, generator=g) > 0.35).float()
+    assert 0 < int(mask.sum()) < B * S
+    keep = mask.reshape(-1).bool()
+    want = R.load_balancing_loss(tuple(l[keep] for l in layers), N, K)
+    got = R.load_balancing_loss(layers, N, K, attention_mask=mask)
+    assert abs(float(got) - float(want)) <= 1e-6 * float(want)
+    plain = R.load_balancing_loss(layers, N, K)
+    assert abs(float(R.load_balancing_loss(layers, N, K, attention_mask=torch.ones(B, S))) - float(plain)) <= 1e-6 * float(plain)
+    assert abs(float(got) - float(plain)) > 1e-4 * float(plain)
+    # dividing by the number of tokens instead of the mask sum scales the loss by (sum m / T)^2
+    frac = float(mask.mean())
+    assert abs(float(got) * frac * frac - float(got)) > 1e-2 * float(got)
+    # gradient flows only into kept tokens
+    lg = tuple(l.clone().requires_grad_(True) for l in layers)
+    R.load_balancing_loss(lg, N, K, attention_mask=mask).backward()
+    for l in lg:
+        assert float(l.grad[~keep].abs().max()) == 0.0 and float(l.grad[keep].abs().max()) > 0.0
