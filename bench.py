@@ -36,12 +36,13 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # counters cannot be collected inside the timed run.
 MIB = float(1 << 20)
 MEASURED_TRAFFIC_BYTES = {
-    "om_merged_mlp_gate_up_fwd": (3220 + 768) * MIB, "om_grouped_gemm_fwd": (1389 + 512) * MIB,
-    "om_grouped_gemm_wgrad": (927 + 256) * MIB, "om_merged_mlp_down_dgrad": (1952 + 512) * MIB,
-    "om_merged_mlp_gate_up_dgrad": (3480 + 512) * MIB, "om_adamw_step": (92125 + 92125) * MIB,
-    "om_merged_mlp_gate_up_fwd_gathered": (3288 + 768) * MIB, "om_grouped_gemm_wgrad_gathered": (989 + 256) * MIB,
-    "om_merged_mlp_gate_up_fwd_weighted": (3241 + 768) * MIB, "om_grouped_gemm_wgrad_gathered_out": (903 + 256) * MIB,
-    "om_merged_mlp_down_dgrad_weighted": (1927 + 523) * MIB,
+    "om_merged_mlp_gate_up_fwd_weighted": (3317 + 768.6) * MIB, "om_grouped_gemm_fwd": (1396.5 + 512) * MIB,
+    "om_merged_mlp_gate_up_dgrad": (3490 + 512) * MIB, "om_merged_mlp_down_dgrad_weighted": (1944.8 + 523.6) * MIB,
+    "om_grouped_gemm_wgrad_gathered": (962.5 + 256) * MIB, "om_grouped_gemm_wgrad_gathered_out": (911.7 + 256) * MIB,
+    "om_adamw_step": (92125 + 92125) * MIB,
+    # entry points a C3 step no longer launches, as measured when it did
+    "om_merged_mlp_gate_up_fwd": (3220 + 768) * MIB, "om_grouped_gemm_wgrad": (927 + 256) * MIB,
+    "om_merged_mlp_down_dgrad": (1952 + 512) * MIB, "om_merged_mlp_gate_up_fwd_gathered": (3288 + 768) * MIB,
 }
 
 GEMM_ENTRY_PRODUCTS = {     # C-ABI entry -> number of [rows x N x K] products per launch
@@ -331,6 +332,69 @@ def bench_other_configs(args, device, with_cpu):
     return out
 
 
+def bench_power_probe(args, device):
+    """Not the metric: the five expert-GEMM entry points of the C3 step called directly on synthetic
+    operands of the C3 shapes (uniformly random routing), once with N(0,1)-like data and once with
+    all-zero activations and weights.  The arithmetic, the loads and the schedule are identical; only
+    the switching activity in the matrix cores differs, so the ratio shows how far the chip's power
+    limit, not the kernel's structure, sets the rate (pair it with `rocprofv3 --pmc GRBM_GUI_ACTIVE`
+    for the engine clock)."""
+    import torch
+    from optimus import _native as n
+    lib = n.lib()
+    T, K, H, I, G = 16384, 8, 2048, 1024, 64
+    TR = T * K
+    g = torch.Generator(device=device).manual_seed(1)
+    e = torch.topk(torch.randn(T, G, device=device, generator=g), K, dim=1).indices.flatten()
+    input_indices = (torch.argsort(e, stable=True) // K).to(torch.int32).contiguous()
+    cum = torch.zeros(G + 1, dtype=torch.int32, device=device)
+    cum[1:] = torch.cumsum(torch.bincount(e, minlength=G), 0)
+    bf = torch.bfloat16
+    out = {}
+    for kind in ("random", "zeros"):
+        mk = (lambda *shape, scale=1.0: (torch.randn(*shape, device=device, generator=g) * scale).to(bf)) \
+            if kind == "random" else (lambda *shape, scale=1.0: torch.zeros(*shape, device=device, dtype=bf))
+        x, dfinal = mk(T, H), mk(T, H)
+        wg, wu, wd = mk(G, I, H, scale=0.02), mk(G, I, H, scale=0.02), mk(G, H, I, scale=0.02)
+        roww = torch.rand(TR, device=device, generator=g) if kind == "random" else torch.zeros(TR, device=device)
+        gb, ub, hb = (torch.empty(TR, I, device=device, dtype=bf) for _ in range(3))
+        dg, du = torch.empty_like(gb), torch.empty_like(gb)
+        y, dx = torch.empty(TR, H, device=device, dtype=bf), torch.empty(TR, H, device=device, dtype=bf)
+        dwg, dwu, dwd = torch.empty_like(wg), torch.empty_like(wu), torch.empty_like(wd)
+        row_dot = torch.empty(I // 64, TR, device=device)
+        P, st = n.ptr, n.stream()
+        calls = [
+            (2, lambda: lib.om_merged_mlp_gate_up_fwd_weighted(P(x), P(input_indices), T, P(wg), P(wu), P(roww), P(gb), P(ub), P(hb), P(cum), TR, G, I, H, 0, st)),
+            (1, lambda: lib.om_grouped_gemm_fwd(P(hb), P(wd), P(y), P(cum), TR, G, H, I, 0, st)),
+            (1, lambda: lib.om_merged_mlp_down_dgrad_weighted(P(dfinal), P(input_indices), T, P(wd), P(gb), P(ub), P(roww), P(dg), P(du), P(row_dot), P(cum), TR, G, I, H, 0, st)),
+            (2, lambda: lib.om_merged_mlp_gate_up_dgrad(P(dg), P(du), P(wg), P(wu), P(dx), P(cum), TR, G, I, H, 0, st)),
+            (1, lambda: lib.om_grouped_gemm_wgrad_gathered(P(dg), P(x), P(input_indices), T, P(dwg), P(cum), TR, G, I, H, 0, st)),
+            (1, lambda: lib.om_grouped_gemm_wgrad_gathered(P(du), P(x), P(input_indices), T, P(dwu), P(cum), TR, G, I, H, 0, st)),
+            (1, lambda: lib.om_grouped_gemm_wgrad_gathered_out(P(dfinal), P(input_indices), T, P(hb), P(dwd), P(cum), TR, G, H, I, 0, st)),
+        ]
+
+        def step():
+            for _, fn in calls:
+                n.check(fn(), "power probe")
+        for _ in range(max(3, args.warmup)):
+            step()
+        torch.cuda.synchronize()
+        a = torch.cuda.Event(enable_timing=True); b = torch.cuda.Event(enable_timing=True)
+        reps = max(5, args.steps)
+        a.record()
+        for _ in range(reps):
+            step()
+        b.record(); torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / reps
+        out[kind] = {"ms_per_nine_products": round(ms, 3),
+                     "tflops": round(9 * 2.0 * TR * H * I / (ms * 1e-3) / 1e12, 1),
+                     "frac_of_peak": round(9 * 2.0 * TR * H * I / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+        del x, dfinal, wg, wu, wd, gb, ub, hb, dg, du, y, dx, dwg, dwu, dwd
+        torch.cuda.empty_cache()
+    out["zeros_over_random"] = round(out["zeros"]["tflops"] / out["random"]["tflops"], 3)
+    return out
+
+
 def cpu_baseline_moe():
     """oracle.moe_layer.olmoe_slow_block (the reference's per-expert loop, fp32) forward+backward on
     1/16 of the C3 tokens with the full expert weights; tokens/s of that run."""
@@ -489,6 +553,10 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baselines")
     ap.add_argument("--skip-adamw", action="store_true", help="leave out the AdamW workload")
     ap.add_argument("--skip-other", action="store_true", help="leave out the C1 / C4 / C5 configurations")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only run four 1 GiB device copies (calibrates the HBM traffic counters)")
+    ap.add_argument("--power-probe", action="store_true",
+                    help="only run the expert GEMMs on random and on all-zero operands (power-limit evidence)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU's hot path; --gpus must be 1 "
@@ -501,6 +569,21 @@ def main():
     from optimus import _native
     _native.lib()
     device = torch.device("cuda:0")
+    if args.power_probe:
+        print(json.dumps({"power_probe": bench_power_probe(args, device), "n_gpus": 1,
+                          "note": "expert GEMM entry points on random vs all-zero operands; not the metric"}))
+        return
+    if args.copy_probe:
+        # a device-to-device copy of known size: what FETCH_SIZE / WRITE_SIZE read for it gives the
+        # factors that turn those counters into bytes
+        n = 1 << 30
+        src = torch.empty(n, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe": {"bytes_per_copy": n, "copies": 4}, "n_gpus": 1}))
+        return
     moe = bench_moe(args, device)
     out = {
         "metric": "olmoe_moe_layer_fwd_bwd_tokens_per_s", "value": round(moe["T"] / (moe["ms_per_step"] * 1e-3), 1),
