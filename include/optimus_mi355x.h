@@ -101,6 +101,19 @@ int om_grad_norm_clip_coef(const float *partials, const int64_t *seg_first_chunk
  * model that the optimizer does not hold, or skip_optimizer_step).  grad 16-byte aligned.       */
 int om_grad_scale(void *grad, int64_t n, int grad_dtype, const float *coef, void *stream);
 
+/* om_shard_clip_multiplier: the clip decision of the sharded optimizer's step
+ * (ShardedMixedPrecisionAdamW.step, optimizers.py:398-432) on the device, so that the step never
+ * reads the norm back.  mode 0 (no process group, :404-405): *value is this shard's gradient norm,
+ * already rounded to the gradient dtype (om_grad_norm_clip_coef's total_norm over one segment), and
+ * the coefficient max_norm / (norm + 1e-6) is evaluated with every op rounded to that dtype.
+ * mode 1 (:399-403): *value is the all-reduced sum of the ranks' squared fp32 shard norms; the norm
+ * and the coefficient are fp32.  *grad_norm receives the norm; *multiplier what
+ * `if clip_coef < 1.0: flat_grad_shard.mul_(clip_coef)` multiplies by: the coefficient rounded to
+ * the gradient dtype (the cast torch applies to a 0-dim device operand) when it is below 1, else 1.
+ * Feed *multiplier to om_adamw_step_clipped / om_grad_scale.  All three are device fp32 scalars. */
+int om_shard_clip_multiplier(const float *value, int mode, int grad_dtype, double max_norm,
+                             float *grad_norm, float *multiplier, void *stream);
+
 /* om_adamw_step with the clip folded in: g = cast(grad * *grad_scale) is what the update uses,
  * i.e. the in-place multiply of clip_grads_with_norm_ (optimizers.py:145/150/154) without its
  * read-modify-write pass over the gradients.  *grad_scale is a device fp32 scalar (the clip_coef

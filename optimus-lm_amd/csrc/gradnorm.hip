@@ -127,6 +127,35 @@ __global__ __launch_bounds__(256) void total_norm_kernel(const float *__restrict
     }
 }
 
+// Clip multiplier of the sharded optimizer (reference optimus/optimizers.py:398-432), one thread.
+//   mode 0  no process group (:404-405): *value is this shard's norm, already rounded to the
+//           gradient dtype, and max_norm / (norm + 1e-6) is evaluated on that 0-dim tensor: the sum,
+//           the reciprocal and the product are each rounded to the gradient dtype;
+//   mode 1  after the all-reduce (:399-403): *value is the sum over the ranks of the squared fp32
+//           shard norms; norm = sqrt(value) and the coefficient are plain fp32.
+// `flat_grad_shard.mul_(clip_coef)` runs only when clip_coef < 1 (:431-432) and, both operands being
+// device tensors, casts the 0-dim coefficient to the gradient dtype before multiplying; hence
+// *multiplier = coef < 1 ? round(coef) : 1 (a NaN coefficient compares false and scales nothing).
+template <typename T>
+__global__ void shard_clip_kernel(const float *__restrict__ value, int mode, float max_norm,
+                                  float *__restrict__ grad_norm, float *__restrict__ multiplier) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    float norm, c;
+    if (mode == 0) {
+        norm = *value;
+        const float x = round_to<T>(norm + 1e-6f);
+        const float r = round_to<T>(1.0f / x);
+        c = round_to<T>(r * max_norm);
+    } else {
+        norm = sqrtf(*value);
+        const float x = norm + 1e-6f;
+        const float r = 1.0f / x;
+        c = r * max_norm;
+    }
+    *grad_norm = norm;
+    *multiplier = c < 1.0f ? round_to<T>(c) : 1.0f;
+}
+
 // grad = cast(float(grad) * *coef), 16 bytes per lane, scalar tail.
 template <typename T>
 __global__ __launch_bounds__(256) void grad_scale_kernel(T *__restrict__ grad, int64_t n,
@@ -168,6 +197,20 @@ extern "C" int om_grad_scale(void *grad, int64_t n, int grad_dtype, const float 
     else
         grad_scale_kernel<float><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(
             static_cast<float *>(grad), n, coef);
+    return om_launch_status();
+}
+
+extern "C" int om_shard_clip_multiplier(const float *value, int mode, int grad_dtype, double max_norm,
+                                        float *grad_norm, float *multiplier, void *stream) {
+    if (grad_dtype != OM_BF16 && grad_dtype != OM_F32) return OM_ERR_DTYPE;
+    if (mode != 0 && mode != 1) return OM_ERR_SHAPE;
+    if (!value || !grad_norm || !multiplier) return OM_ERR_NULL;
+    hipStream_t st = om_stream(stream);
+    const float mx = static_cast<float>(max_norm);
+    if (grad_dtype == OM_BF16)
+        shard_clip_kernel<uint16_t><<<dim3(1), dim3(64), 0, st>>>(value, mode, mx, grad_norm, multiplier);
+    else
+        shard_clip_kernel<float><<<dim3(1), dim3(64), 0, st>>>(value, mode, mx, grad_norm, multiplier);
     return om_launch_status();
 }
 

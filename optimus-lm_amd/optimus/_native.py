@@ -32,6 +32,7 @@ SIGNATURES = {
     "om_grad_norm_clip_coef": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_double, c_void_p, c_void_p,
                                        c_void_p, c_void_p]),
     "om_grad_scale": (c_int, [c_void_p, c_i64, c_int, c_void_p, c_void_p]),
+    "om_shard_clip_multiplier": (c_int, [c_void_p, c_int, c_int, c_double, c_void_p, c_void_p, c_void_p]),
     "om_adamw_step_clipped": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64,
                                       c_double, c_double, c_double, c_double, c_double, c_i64, c_int,
                                       c_void_p, c_int, c_void_p]),

@@ -1,5 +1,5 @@
-"""optimus.optimizers — MixedPrecisionAdamW with the reference's interface
-(optimus/optimizers.py:19-225) and a single-pass HIP kernel for the update.
+"""optimus.optimizers — MixedPrecisionAdamW and ShardedMixedPrecisionAdamW with the reference's
+interfaces (optimus/optimizers.py:19-225, :227-522) and a single-pass HIP kernel for the update.
 
 All parameters, gradients and optimizer states live in five flat buffers: `flat_param` and
 `flat_grad` in the model dtype, `flat_exp_avg`, `flat_exp_avg_sq` and `flat_fp32_master_param`
@@ -170,6 +170,236 @@ class MixedPrecisionAdamW(Optimizer):
     def load_state_dict(self, opt_state_dict):
         for key in _STATE_KEYS:
             getattr(self, key).copy_(opt_state_dict[key].to(self.device))
+        self.step_id = opt_state_dict["step_id"]
+
+
+_SHARD_STATE_KEYS = ("flat_exp_avg_shard", "flat_exp_avg_sq_shard", "flat_fp32_master_param_shard")
+_ALLREDUCE_PART = 128 * 1024 * 1024      # elements per call of the chunked all-reduce (optimizers.py:11-17)
+
+
+class ProcessGroupExchange:
+    """The three collectives of the sharded step, made through torch.distributed exactly where the
+    reference makes them (optimus/optimizers.py:362-375, :402, :481-494).  Without an initialised
+    process group `active()` is false and the step is the single-process one."""
+
+    def active(self):
+        return torch.distributed.is_available() and torch.distributed.is_initialized()
+
+    def reduce_scatter(self, shard, full, group):
+        torch.distributed.reduce_scatter_tensor(shard, full, group=group)
+
+    def all_reduce(self, tensor, group=None):
+        torch.distributed.all_reduce(tensor, group=group)
+
+    def all_gather(self, full, shard, group):
+        torch.distributed.all_gather_into_tensor(full, shard, group=group)
+
+
+class ShardedMixedPrecisionAdamW(Optimizer):
+    """AdamW whose fp32 master weights and moments exist only for this rank's shard of the flat
+    buffer; interface of the reference class (optimus/optimizers.py:227-522).
+
+    `flat_param` / `flat_grad` span `num_shards * shard_size` elements in the model dtype (the
+    parameters back to back, then zero padding up to a multiple of `shard_divisible_by` per shard);
+    `flat_param_shard` / `flat_grad_shard` are this rank's slices and `flat_exp_avg_shard`,
+    `flat_exp_avg_sq_shard`, `flat_fp32_master_param_shard` its float32 states.  One step is: gradient
+    exchange (reduce-scatter, or all-reduce), the shard's norm, the all-reduced total norm, the clip
+    and the AdamW update of the shard in ONE kernel pass, parameter exchange (all-gather, or
+    all-reduce).  Norm, coefficient and clip decision stay on the device: the reference's
+    `if clip_coef < 1.0` (:431) reads the norm back every step, here a one-thread kernel turns it into
+    a multiplier (1 when nothing is to be clipped) that the update kernel applies.
+
+    Kept from the reference: one parameter group, `device` given.  Beyond it: no expert or tensor
+    parallelism (their replicated-parameter rescaling needs model hooks outside this path);
+    `shard_size` a multiple of 8; in float32 mode the master shard is `flat_param_shard` itself (the
+    reference keeps a second float32 copy with the same values)."""
+
+    def __init__(self,
+                 params, model,
+                 lr=0.001,
+                 betas=(0.9, 0.999),
+                 eps=1e-08,
+                 weight_decay=0.01, warmup_steps=0,
+                 dtype=torch.float32, device=None,
+                 num_shards=1, shard_id=0, group=None,
+                 opt_disable_delayed_grad_clipping=False,
+                 profiler=None,
+                 tensor_parallelism=1, tp_ind=0, tp_group=None,
+                 expert_parallelism=1, ep_ind=0, ep_group=None,
+                 dpep_ind=0, dpep_group=None,
+                 shard_divisible_by=512,
+                 opt_use_chunked_allreduce=False,
+                 opt_use_allreduce_for_grad_acc=False,
+                 opt_use_allreduce_for_param_gather=False,
+                 skip_optimizer_step=False,
+                 disable_optimizer_state_checkpointing=False,
+                 skip_optimizer_step_weight_update=False):
+        super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
+        if device is None:
+            raise AssertionError("ShardedMixedPrecisionAdamW needs the device of the flat buffers")
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError("ShardedMixedPrecisionAdamW: dtype must be torch.float32 or torch.bfloat16")
+        if len(self.param_groups) != 1:
+            raise AssertionError("Only one parameter group is supported")
+        if expert_parallelism != 1 or tensor_parallelism != 1:
+            raise AssertionError("expert / tensor parallelism are outside the single-GPU hot path")
+        if not 0 <= shard_id < num_shards:
+            raise ValueError(f"shard_id {shard_id} outside [0, {num_shards})")
+        self.opt_key = "shard"
+        for name, value in (("model", model), ("warmup_steps", warmup_steps), ("dtype", dtype),
+                            ("device", device), ("profiler", profiler),
+                            ("opt_disable_delayed_grad_clipping", opt_disable_delayed_grad_clipping),
+                            ("tensor_parallelism", tensor_parallelism), ("tp_ind", tp_ind),
+                            ("tp_group", tp_group), ("expert_parallelism", expert_parallelism),
+                            ("ep_ind", ep_ind), ("ep_group", ep_group), ("dpep_ind", dpep_ind),
+                            ("dpep_group", dpep_group),
+                            ("data_parallelism", num_shards), ("dp_ind", shard_id), ("dp_group", group),
+                            ("shard_divisible_by", shard_divisible_by),
+                            ("opt_use_chunked_allreduce", opt_use_chunked_allreduce),
+                            ("opt_use_allreduce_for_grad_acc", opt_use_allreduce_for_grad_acc),
+                            ("opt_use_allreduce_for_param_gather", opt_use_allreduce_for_param_gather),
+                            ("skip_optimizer_step", skip_optimizer_step),
+                            ("disable_optimizer_state_checkpointing", disable_optimizer_state_checkpointing),
+                            ("skip_optimizer_step_weight_update", skip_optimizer_step_weight_update)):
+            setattr(self, name, value)
+        self.step_id = 0
+        self.dump_weight_gradients = False     # a debugging switch the reference's trainer sets
+        self.exchange = ProcessGroupExchange()
+
+        self.param_list = list(self.param_groups[0]["params"])
+        self.param_sizes, self.param_start_inds, offset = [], [], 0
+        for p in self.param_list:
+            self.param_start_inds.append(offset)
+            self.param_sizes.append(p.numel())
+            offset += p.numel()
+        self.flat_param_size = offset
+
+        # every shard holds a whole number of `shard_divisible_by` blocks (optimizers.py:297-298)
+        block = num_shards * shard_divisible_by
+        self.shard_size = (offset + block - 1) // block * shard_divisible_by
+        self.flat_buffer_size = num_shards * self.shard_size
+        if self.shard_size % 8:
+            raise ValueError("shard_size must be a multiple of 8 elements (16-byte aligned shard views); "
+                             f"got {self.shard_size} from shard_divisible_by={shard_divisible_by}")
+
+        self.flat_param = torch.zeros(self.flat_buffer_size, dtype=dtype, device=device)
+        self.flat_grad = torch.zeros(self.flat_buffer_size, dtype=dtype, device=device)
+        lo = shard_id * self.shard_size
+        self.flat_param_shard = self.flat_param.narrow(0, lo, self.shard_size)
+        self.flat_grad_shard = self.flat_grad.narrow(0, lo, self.shard_size)
+
+        if self.param_list:
+            pad = [self.flat_buffer_size - offset] if self.flat_buffer_size > offset else []
+            slices = self.flat_param.split(self.param_sizes + pad)
+            grad_slices = self.flat_grad.split(self.param_sizes + pad)
+            with torch.no_grad():
+                for p, dst, gdst in zip(self.param_list, slices, grad_slices):
+                    dst = dst.view(p.shape)
+                    dst.copy_(p.data)
+                    p.data = dst
+                    p.grad = gdst.view(p.shape)
+
+        def state():
+            return torch.zeros(self.shard_size, dtype=torch.float32, device=device)
+
+        if skip_optimizer_step:
+            self.flat_exp_avg_shard = self.flat_exp_avg_sq_shard = self.flat_fp32_master_param_shard = None
+        else:
+            self.flat_exp_avg_shard, self.flat_exp_avg_sq_shard = state(), state()
+            self.flat_fp32_master_param_shard = self.flat_param_shard if dtype == torch.float32 \
+                else self.flat_param_shard.to(torch.float32)
+        self._norm_plan = GradNormPlan([0], [self.shard_size], device) if self.shard_size else None
+        self._clip = torch.zeros(2, dtype=torch.float32, device=device)    # grad norm, clip multiplier
+
+    def zero_grad(self):
+        self.flat_grad.zero_()
+
+    def _all_reduce_flat(self, tensor):
+        parts = tensor.split(_ALLREDUCE_PART) if self.opt_use_chunked_allreduce else (tensor,)
+        for part in parts:
+            self.exchange.all_reduce(part, self.dp_group)
+
+    def _accumulate_gradients(self, distributed):
+        """Sum over the data-parallel ranks and average (optimizers.py:361-375)."""
+        if not distributed or self.data_parallelism == 1:
+            return
+        if self.opt_use_allreduce_for_grad_acc:
+            self._all_reduce_flat(self.flat_grad)
+            self.flat_grad.div_(self.data_parallelism)
+        else:
+            self.exchange.reduce_scatter(self.flat_grad_shard, self.flat_grad, self.dp_group)
+            self.flat_grad_shard.div_(self.data_parallelism)
+
+    def shard_grad_norm(self):
+        """Norm of this rank's gradient shard, rounded to the gradient dtype like
+        torch.nn.utils.get_total_norm(flat_grad_shard) (optimizers.py:398); a 0-dim float32 device
+        tensor that the next call overwrites."""
+        return self._norm_plan.run(self.flat_grad_shard)[0]
+
+    def _norm_and_multiplier(self, distributed):
+        """optimizers.py:398-405 and :430-431: returns (grad_norm, multiplier) as device scalars."""
+        shard_norm = self.shard_grad_norm()
+        if distributed:
+            value = shard_norm * shard_norm              # torch.pow(norm.float(), 2)
+            self.exchange.all_reduce(value)              # over every rank of the job, like :402
+        else:
+            value = shard_norm
+        _n.check(_n.lib().om_shard_clip_multiplier(
+            _n.ptr(value), 1 if distributed else 0, _n.dtype_code(self.flat_grad), 1.0,
+            _n.ptr(self._clip), _n.ptr(self._clip) + 4, _n.stream()), "om_shard_clip_multiplier")
+        return self._clip[0], self._clip[1:2]
+
+    def _gather_parameters(self, distributed):
+        """Every rank ends the step with all updated parameters (optimizers.py:481-494)."""
+        exchange = distributed and self.data_parallelism > 1
+        if not self.opt_use_allreduce_for_param_gather:
+            if exchange:
+                self.exchange.all_gather(self.flat_param, self.flat_param_shard, self.dp_group)
+            return
+        lo = self.dp_ind * self.shard_size
+        self.flat_param[:lo].zero_()
+        self.flat_param[lo + self.shard_size:].zero_()
+        if exchange:
+            self._all_reduce_flat(self.flat_param)
+
+    def step(self, closure=None):
+        if self.dump_weight_gradients:
+            raise NotImplementedError("dump_weight_gradients is a debugging aid outside this path")
+        distributed = self.exchange.active()
+        with record_pcl_function("4opt-step_1gradacc"):
+            self._accumulate_gradients(distributed)
+        if self.shard_size == 0:
+            self.step_id += 1
+            return torch.zeros((), dtype=torch.float32 if distributed else self.dtype, device=self.device)
+        with record_pcl_function("4opt-step_3global-gradnorm"):
+            grad_norm, multiplier = self._norm_and_multiplier(distributed)
+        clip_now = self.opt_disable_delayed_grad_clipping or (self.step_id >= self.warmup_steps)
+        with record_pcl_function("4opt-step_5compute"):
+            if not (self.skip_optimizer_step or self.skip_optimizer_step_weight_update):
+                group = self.param_groups[0]
+                beta1, beta2 = self.defaults["betas"]
+                adamw_step_(self.flat_param_shard, self.flat_grad_shard, self.flat_fp32_master_param_shard,
+                            self.flat_exp_avg_shard, self.flat_exp_avg_sq_shard, self.step_id + 1,
+                            group["lr"], beta1, beta2, self.defaults["eps"], self.defaults["weight_decay"],
+                            grad_scale=multiplier if clip_now else None, store_scaled_grad=True)
+            elif clip_now:
+                scale_grad_(self.flat_grad_shard, multiplier)
+        self._gather_parameters(distributed)
+        self.step_id += 1
+        # a fresh tensor: float32 after the all-reduce, the gradient dtype without a process group
+        return grad_norm.to(torch.float32 if distributed else self.dtype, copy=True)
+
+    def state_dict(self):
+        state = {"step_id": self.step_id}
+        if not self.disable_optimizer_state_checkpointing:
+            for key in _SHARD_STATE_KEYS:
+                state[key] = getattr(self, key)
+        return state
+
+    def load_state_dict(self, opt_state_dict):
+        for key in _SHARD_STATE_KEYS:
+            if key in opt_state_dict:
+                getattr(self, key).copy_(opt_state_dict[key])
         self.step_id = opt_state_dict["step_id"]
 
 

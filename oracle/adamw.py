@@ -3,6 +3,9 @@
 adamw_step_torch   — the reference's chunked sequence of torch elementwise ops,
                      optimus/optimizers.py:162-205, on CPU tensors.  This is the "port" that
                      bench.py times as cpu_baseline for the AdamW workload.
+sharded_clip_and_step_torch — ShardedMixedPrecisionAdamW.step from the accumulated gradient shards
+                     on (optimus/optimizers.py:398-479) for all ranks at once, collectives replaced
+                     by their definitions.
 The scalar C versions (fp32 op-by-op and fp64) are in oracle/adamw_oracle.c via oracle/clib.py.
 """
 import math
@@ -45,3 +48,36 @@ def grad_norm_and_clip_torch(grads, clip, max_norm=1.0):
             h.grad = g
         torch.nn.utils.clip_grads_with_norm_(holders, max_norm, total)           # :148
     return total
+
+
+def sharded_clip_and_step_torch(grad_shards, param_shards, master_shards, exp_avg_shards, exp_avg_sq_shards,
+                                step_id, lr, betas, eps, weight_decay, clip, process_group, max_norm=1.0):
+    """ShardedMixedPrecisionAdamW.step (optimus/optimizers.py:398-479) for every rank of a job at
+    once, on CPU tensors, in place; rank r owns element r of each list.  The gradient shards are
+    taken as already accumulated (the reduce-scatter's summation order belongs to the collective).
+    `process_group` False is the single-process branch (:404-405; one rank only).
+    Two things are made explicit that the device run of the reference does implicitly:
+      * all_reduce(sum) of the squared norms = the ranks' values added in rank order;
+      * `flat_grad_shard.mul_(clip_coef)` with both operands on the device casts the 0-dim float32
+        coefficient to the gradient dtype before multiplying (on CPU tensors torch would take a 0-dim
+        operand as an exact scalar), hence `.to(g.dtype)` below.
+    Returns grad_norm as the reference's step does."""
+    norms = [torch.nn.utils.get_total_norm(g) for g in grad_shards]               # :398
+    if process_group:
+        total = None
+        for n in norms:
+            sq = torch.pow(n.to(torch.float32), 2)                                # :400-401
+            total = sq if total is None else total + sq                           # :402
+        grad_norm = torch.sqrt(total)                                             # :403
+    else:
+        assert len(grad_shards) == 1
+        grad_norm = norms[0]                                                      # :405
+    if clip:
+        clip_coef = max_norm / (grad_norm + 1e-6)                                 # :430
+        if clip_coef < 1.0:                                                       # :431
+            for g in grad_shards:
+                g.mul_(clip_coef.to(g.dtype))                                     # :432
+    for r in range(len(grad_shards)):                                             # :434-479
+        adamw_step_torch(param_shards[r], grad_shards[r], master_shards[r], exp_avg_shards[r],
+                         exp_avg_sq_shards[r], step_id, lr, betas, eps, weight_decay)
+    return grad_norm

@@ -173,3 +173,38 @@ void orc_scale_grads_bf16(bf16_t *grad, int64_t n, float coef) {
 void orc_scale_grads_f32(float *grad, int64_t n, float coef) {
     for (int64_t i = 0; i < n; i++) grad[i] = grad[i] * coef;
 }
+
+/*
+ * Clip decision of the sharded optimizer, ShardedMixedPrecisionAdamW.step, optimizers.py:398-432.
+ * The shard's norm is get_total_norm of ONE tensor (the rank's slice of the flat gradient), i.e.
+ * bf16( sqrt( sum g^2 ) ) for bf16 gradients (orc_grad_norm_clip_* with a single segment gives it).
+ *   mode 0, no process group (:404-405): grad_norm is that 0-dim tensor in the gradient dtype, and
+ *     clip_coef = max_norm / (grad_norm + 1e-6) = (grad_norm + 1e-6).reciprocal() * max_norm is
+ *     evaluated in that dtype: sum, reciprocal and product each rounded.
+ *   mode 1, process group (:399-403): `value` is the all-reduced sum of float(norm)^2 over the ranks;
+ *     grad_norm = sqrt(value), clip_coef = 1 / (grad_norm + 1e-6) * max_norm, all fp32.
+ * :431-432 multiplies the shard in place only if clip_coef < 1.  Both operands of that mul_ live on
+ * the device, so torch casts the 0-dim coefficient to the gradient dtype before the multiply (a CPU
+ * 0-dim operand would be taken as an exact scalar instead; the reference's norm is a device tensor).
+ * `multiplier` is therefore round(clip_coef) when clip_coef < 1 and 1 otherwise (NaN included).
+ */
+static float round_bf16(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+void orc_shard_clip_multiplier(float value, int mode, int grad_is_bf16, double max_norm,
+                               float *grad_norm, float *multiplier) {
+    float norm, c;
+    if (mode == 0) {
+        norm = value;
+        if (grad_is_bf16) {
+            float x = round_bf16(norm + 1e-6f);
+            float r = round_bf16(1.0f / x);
+            c = round_bf16(r * (float)max_norm);
+        } else {
+            c = (1.0f / (norm + 1e-6f)) * (float)max_norm;
+        }
+    } else {
+        norm = sqrtf(value);
+        c = (1.0f / (norm + 1e-6f)) * (float)max_norm;
+    }
+    *grad_norm = norm;
+    *multiplier = (c < 1.0f) ? (grad_is_bf16 ? round_bf16(c) : c) : 1.0f;
+}

@@ -236,3 +236,13 @@ def scale_grads(grad, coef):
     assert grad.flags.c_contiguous and grad.dtype in (np.uint16, np.float32)
     fn = lib().orc_scale_grads_bf16 if grad.dtype == np.uint16 else lib().orc_scale_grads_f32
     fn(_p(grad), I64(grad.size), ctypes.c_float(coef))
+
+
+def shard_clip_multiplier(value, mode, grad_is_bf16, max_norm=1.0):
+    """(grad_norm, multiplier) of the sharded optimizer's clip decision; `value` is the shard norm
+    (mode 0) or the summed squared shard norms (mode 1)."""
+    norm = np.zeros(1, dtype=np.float32)
+    mult = np.zeros(1, dtype=np.float32)
+    lib().orc_shard_clip_multiplier(ctypes.c_float(value), ctypes.c_int(mode), ctypes.c_int(int(grad_is_bf16)),
+                                    F64(max_norm), _p(norm), _p(mult))
+    return float(norm[0]), float(mult[0])

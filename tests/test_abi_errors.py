@@ -85,6 +85,10 @@ def test_routers(lib):
     assert lib.om_grad_scale(P, 100, BF16, None, None) == NULL
     assert lib.om_grad_scale(ODD, 100, BF16, P, None) == ALIGN
     assert lib.om_grad_scale(None, 0, BF16, None, None) == OK
+    assert lib.om_shard_clip_multiplier(P, 0, 7, 1.0, P, P, None) == DTYPE
+    assert lib.om_shard_clip_multiplier(P, 2, BF16, 1.0, P, P, None) == SHAPE
+    assert lib.om_shard_clip_multiplier(None, 0, BF16, 1.0, P, P, None) == NULL
+    assert lib.om_shard_clip_multiplier(P, 1, BF16, 1.0, P, None, None) == NULL
     assert lib.om_adamw_traffic_probe(P, P, P, None, P, 1024, None) == NULL
     assert lib.om_router_balance_stats_masked(P, 7, P, 100, 64, 8, P, P, P, 1 << 20, None) == DTYPE
     assert lib.om_router_balance_stats_masked(P, F32, None, 100, 64, 65, P, P, P, 1 << 20, None) == SHAPE
