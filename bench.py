@@ -502,7 +502,30 @@ def bench_adamw(args, device):
         "clipped_step_no_store_gb_per_s": round(28.0 * n / t_clip[False] / 1e9, 1),
         "note": "norm pass reads 2 B/param; clipped step = 28 B/param + 2 B/param when the scaled "
                 "gradient is stored back; 54 parameter slices, 65536-element chunks"}
-    del st, plan
+    # One rank's share of the same buffers under 8-way sharding (ShardedMixedPrecisionAdamW.step,
+    # reference optimizers.py:398-479, without the collectives): norm of the shard, clip decision on
+    # the device, update with the clip folded in and the clipped gradient stored back.
+    shard = -(-n // (8 * 512)) * 512
+    sh = {k: v[:shard] for k, v in st.items()}
+    shard_plan = GradNormPlan([0], [shard], device)
+    clip_buf = torch.zeros(2, dtype=torch.float32, device=device)
+
+    def shard_step():
+        norm = shard_plan.run(sh["grad"])[0]
+        _native.check(_native.lib().om_shard_clip_multiplier(
+            _native.ptr(norm), 0, _native.OM_BF16, 1.0, _native.ptr(clip_buf), _native.ptr(clip_buf) + 4,
+            _native.stream()), "om_shard_clip_multiplier")
+        adamw_step_(sh["param"], sh["grad"], sh["master"], sh["exp_avg"], sh["exp_avg_sq"], hp["step_id"] + 1,
+                    hp["lr"], hp["betas"][0], hp["betas"][1], hp["eps"], hp["weight_decay"],
+                    grad_scale=clip_buf[1:2], store_scaled_grad=True)
+    t_shard = timed(shard_step, ("om_grad_sumsq", "om_grad_norm_clip_coef", "om_shard_clip_multiplier",
+                                 "om_adamw_step_clipped"))
+    sharded = {"what": "one rank's shard of C2 under 8-way sharding: shard norm, device-side clip decision, "
+                       "clipped update storing the scaled gradient (4 launches, 32 B/param)",
+               "shard_params": shard, "ms": round(t_shard * 1e3, 3),
+               "gb_per_s": round(32.0 * shard / t_shard / 1e9, 1),
+               "frac_of_peak": round(32.0 * shard / t_shard / 1e9 / PEAK_HBM_GBS, 4)}
+    del st, sh, plan, shard_plan
     torch.cuda.empty_cache()
     return {"metric": "adamw_step_hbm_gb_per_s", "value": round(gbs, 1), "unit": "GB/s",
             "ms_per_step": round((t1 - t0) * 1e3 / steps, 3), "steps": steps, "dtype": "f32",
@@ -517,7 +540,7 @@ def bench_adamw(args, device):
                                      "the arithmetic, same buffers, same process",
                              "gb_per_s": round(probe_gbs, 1), "frac_of_peak": round(probe_gbs / PEAK_HBM_GBS, 4),
                              "update_over_probe": round(gbs / probe_gbs, 4)}},
-            "grad_clip": grad_clip}
+            "grad_clip": grad_clip, "sharded_step": sharded}
 
 
 def cpu_baseline_adamw():
