@@ -189,6 +189,29 @@ def _timed_steps(step, warmup, steps):
     return ms, {k: v / steps for k, v in per.items()}
 
 
+def _graph_replay_ms(step, steps):
+    """ms per replay of step() recorded once into a HIP graph (torch.cuda.CUDAGraph): what the same
+    kernels take without the host's per-launch work.  step() must allocate its gradients itself."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
 def bench_other_configs(args, device, with_cpu):
     """The other MoE configurations of BASELINE.json, each as whole-block forward+backward on the GPU:
     C1 (tiny, run in bf16 here; its float32 CPU reference path timed in full beside it), C4 (skewed
@@ -236,9 +259,13 @@ def bench_other_configs(args, device, with_cpu):
         o.backward(dout)
     ms, per = _timed_steps(step_c1, args.warmup, steps)
     flops = 18.0 * c["T"] * c["K"] * c["H"] * c["I"]
+    graph_ms = _graph_replay_ms(step_c1, max(steps, 20))
     out["C1"] = entry(c["T"], ms, per, flops, extra={
+        "graph_replay_ms_per_step": round(graph_ms, 4),
+        "graph_replay_tokens_per_s": round(c["T"] / (graph_ms * 1e-3), 1),
         "workload": "C1 tiny MoE layer fwd+bwd (2048 tokens, hidden 256, 8 experts, top-2 renormalised, ffn 512), "
-                    "bf16 on the GPU; about 25 launches, launch-bound"})
+                    "bf16 on the GPU; about 25 launches, launch-bound when launched from Python "
+                    "(ms_per_step); graph_replay_* is the same step recorded once into a HIP graph"})
     if with_cpu:
         from oracle import moe_layer as L
         cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
@@ -280,7 +307,9 @@ def bench_other_configs(args, device, with_cpu):
     with torch.no_grad():
         _, e = SoftmaxTopkRouterFunction.apply(logits, c["K"], False, torch.bfloat16)
         counts = torch.bincount(e.flatten(), minlength=c["N"])
+    graph_ms = _graph_replay_ms(step_c4, max(steps, 20))
     out["C4"] = entry(c["T"], ms, per, flops, wbytes, extra={
+        "graph_replay_ms_per_step": round(graph_ms, 4),
         "workload": "C4 OLMoE-shape layer under Zipf(1.2) routing, 512 tokens (router on injected logits, "
                     "permutation, expert GEMMs, combine; fwd+bwd)",
         "rows_per_expert": {"min": int(counts.min()), "median": int(counts.median()), "max": int(counts.max()),
