@@ -289,13 +289,13 @@ __global__ __launch_bounds__(256) void gate_dgrad_kernel(const float *__restrict
             const int64_t o = tt * H + h;
             if (base) {
                 float a[8], g[8];
-                Elem<uint16_t>::unpack(*reinterpret_cast<const u32x4 *>(base + o), a);
+                Elem<uint16_t>::unpack(__builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + o)), a);   // read once
                 Elem<uint16_t>::unpack(v, g);
 #pragma unroll
                 for (int i = 0; i < 8; i++) a[i] = a[i] + g[i];
                 v = Elem<uint16_t>::pack(a);
             }
-            *reinterpret_cast<u32x4 *>(out + o) = v;
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out + o));
         }
     }
 }

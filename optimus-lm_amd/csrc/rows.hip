@@ -58,6 +58,9 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
         // The token's row numbers and weights are fetched once, 64 at a time, one per lane, and
         // handed round with lane reads: the row loads then depend on no other load, and the four
         // column chunks a lane owns (4 KB of a row per pass) are in flight together.
+        // Rows and result stream past the caches (nontemporal): measured 121 -> 99 us for 131072 rows
+        // of 2048 bf16 (5.0 -> 6.1 TB/s); single-wavefront blocks or fewer resident wavefronts, which
+        // help the AdamW streams, change nothing here.
         constexpr int CH = 4;
         const int64_t nv = E / V;
         for (int64_t c0 = 0; c0 < nv; c0 += 64 * CH) {
@@ -82,7 +85,7 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
 #pragma unroll
                     for (int u = 0; u < CH; u++) {
                         const int64_t c = c0 + u * 64 + lane;
-                        if (c < nv) q[u] = src[c];
+                        if (c < nv) q[u] = __builtin_nontemporal_load(src + c);   // every row is read once
                     }
 #pragma unroll
                     for (int u = 0; u < CH; u++) {
@@ -101,11 +104,11 @@ __global__ __launch_bounds__(256) void token_reduce_kernel(
                 if (c >= nv) continue;
                 if (res) {
                     float r[V];
-                    Elem<T>::unpack(reinterpret_cast<const u32x4 *>(res)[c], r);
+                    Elem<T>::unpack(__builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(res) + c), r);
 #pragma unroll
                     for (int j = 0; j < V; j++) acc[u][j] = r[j] + round_as<T>(acc[u][j]);
                 }
-                reinterpret_cast<u32x4 *>(dst)[c] = Elem<T>::pack(acc[u]);
+                __builtin_nontemporal_store(Elem<T>::pack(acc[u]), reinterpret_cast<u32x4 *>(dst) + c);
             }
         }
     } else {
