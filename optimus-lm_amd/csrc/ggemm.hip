@@ -861,8 +861,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                 const int64_t m = m0 + q / CPRW;
                 if (m < e_row_end) {
                     const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
-                    gq[it] = *reinterpret_cast<const u32x4 *>(p.G + o);
-                    uq[it] = *reinterpret_cast<const u32x4 *>(p.U + o);
+                    // g and u have no reader after this one: keep them out of the caches (-1 to -3 %)
+                    gq[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.G + o));
+                    uq[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.U + o));
                 }
             }
 #pragma unroll
