@@ -212,7 +212,7 @@ def _graph_replay_ms(step, steps):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
-def bench_other_configs(args, device, with_cpu):
+def bench_other_configs(args, device, with_cpu, only=None):
     """The other MoE configurations of BASELINE.json, each as whole-block forward+backward on the GPU:
     C1 (tiny, run in bf16 here; its float32 CPU reference path timed in full beside it), C4 (skewed
     small batch on injected router logits) and C5 (one rank's share of a DeepSeek-V3 layer).  For the
@@ -245,119 +245,122 @@ def bench_other_configs(args, device, with_cpu):
         return e
 
     # ---- C1 -----------------------------------------------------------------------------------
-    inp = sc.moe_inputs("C1")
-    c = inp["cfg"]
-    blk = build_block(inp, device)
-    x = inp["x"].to(device).view(1, c["T"], c["H"]).requires_grad_(True)
-    dout = inp["dout"].to(device).view_as(x)
+    if only in (None, "C1"):
+        inp = sc.moe_inputs("C1")
+        c = inp["cfg"]
+        blk = build_block(inp, device)
+        x = inp["x"].to(device).view(1, c["T"], c["H"]).requires_grad_(True)
+        dout = inp["dout"].to(device).view_as(x)
 
-    def step_c1():
-        for p in blk.parameters():
-            p.grad = None
-        x.grad = None
-        o, _ = blk(x)
-        o.backward(dout)
-    ms, per = _timed_steps(step_c1, args.warmup, steps)
-    flops = 18.0 * c["T"] * c["K"] * c["H"] * c["I"]
-    graph_ms = _graph_replay_ms(step_c1, max(steps, 20))
-    out["C1"] = entry(c["T"], ms, per, flops, extra={
-        "graph_replay_ms_per_step": round(graph_ms, 4),
-        "graph_replay_tokens_per_s": round(c["T"] / (graph_ms * 1e-3), 1),
-        "workload": "C1 tiny MoE layer fwd+bwd (2048 tokens, hidden 256, 8 experts, top-2 renormalised, ffn 512), "
-                    "bf16 on the GPU; about 25 launches, launch-bound when launched from Python "
-                    "(ms_per_step); graph_replay_* is the same step recorded once into a HIP graph"})
-    if with_cpu:
-        from oracle import moe_layer as L
-        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
-        torch.set_num_threads(cores)
-        t = {k: inp[k].float().requires_grad_(True) for k in ("x", "gate_w", "w_gate", "w_up", "w_down")}
-        best = None
-        for _ in range(3):
-            for v in t.values():
-                v.grad = None
-            t0 = time.perf_counter()
-            o, _ = L.olmoe_slow_block(t["x"], t["gate_w"], t["w_gate"], t["w_up"], t["w_down"], c["K"], True)
-            o.backward(inp["dout"].float())
-            dt = time.perf_counter() - t0
-            best = dt if best is None else min(best, dt)
-        out["C1"]["cpu_baseline"] = {"value": round(c["T"] / best, 1), "unit": "tokens/s", "cores": cores,
-                                     "kind": "port", "sample": f"all 2048 tokens, float32, best of 3 ({best * 1e3:.1f} ms)"}
-    del blk, x, dout
+        def step_c1():
+            for p in blk.parameters():
+                p.grad = None
+            x.grad = None
+            o, _ = blk(x)
+            o.backward(dout)
+        ms, per = _timed_steps(step_c1, args.warmup, steps)
+        flops = 18.0 * c["T"] * c["K"] * c["H"] * c["I"]
+        graph_ms = _graph_replay_ms(step_c1, max(steps, 20))
+        out["C1"] = entry(c["T"], ms, per, flops, extra={
+            "graph_replay_ms_per_step": round(graph_ms, 4),
+            "graph_replay_tokens_per_s": round(c["T"] / (graph_ms * 1e-3), 1),
+            "workload": "C1 tiny MoE layer fwd+bwd (2048 tokens, hidden 256, 8 experts, top-2 renormalised, ffn 512), "
+                        "bf16 on the GPU; about 25 launches, launch-bound when launched from Python "
+                        "(ms_per_step); graph_replay_* is the same step recorded once into a HIP graph"})
+        if with_cpu:
+            from oracle import moe_layer as L
+            cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+            torch.set_num_threads(cores)
+            t = {k: inp[k].float().requires_grad_(True) for k in ("x", "gate_w", "w_gate", "w_up", "w_down")}
+            best = None
+            for _ in range(3):
+                for v in t.values():
+                    v.grad = None
+                t0 = time.perf_counter()
+                o, _ = L.olmoe_slow_block(t["x"], t["gate_w"], t["w_gate"], t["w_up"], t["w_down"], c["K"], True)
+                o.backward(inp["dout"].float())
+                dt = time.perf_counter() - t0
+                best = dt if best is None else min(best, dt)
+            out["C1"]["cpu_baseline"] = {"value": round(c["T"] / best, 1), "unit": "tokens/s", "cores": cores,
+                                         "kind": "port", "sample": f"all 2048 tokens, float32, best of 3 ({best * 1e3:.1f} ms)"}
+        del blk, x, dout
 
     # ---- C4 -----------------------------------------------------------------------------------
-    inp = sc.moe_inputs("C4")
-    c = inp["cfg"]
-    logits = inp["logits"].to(device)
-    t = {k: inp[k].to(device).requires_grad_(True) for k in ("x", "w_gate", "w_up", "w_down")}
-    dout = inp["dout"].to(device)
-    routed = lambda hs, rw, ii, cum_ep, oi, si, cum, res: RoutedMLPFunction.apply(
-        hs, rw, ii, cum_ep, oi, si, cum, res, True, t["w_gate"], t["w_up"], t["w_down"])
-    fn = lambda gi, cum: MergedMLPFunction.apply(gi, t["w_gate"], t["w_up"], t["w_down"], cum)
+    if only in (None, "C4"):
+        inp = sc.moe_inputs("C4")
+        c = inp["cfg"]
+        logits = inp["logits"].to(device)
+        t = {k: inp[k].to(device).requires_grad_(True) for k in ("x", "w_gate", "w_up", "w_down")}
+        dout = inp["dout"].to(device)
+        routed = lambda hs, rw, ii, cum_ep, oi, si, cum, res: RoutedMLPFunction.apply(
+            hs, rw, ii, cum_ep, oi, si, cum, res, True, t["w_gate"], t["w_up"], t["w_down"])
+        fn = lambda gi, cum: MergedMLPFunction.apply(gi, t["w_gate"], t["w_up"], t["w_down"], cum)
 
-    def step_c4():
-        for v in t.values():
-            v.grad = None
-        w, e = SoftmaxTopkRouterFunction.apply(logits, c["K"], False, torch.bfloat16)
-        o = expert_computation(t["x"], w.detach().requires_grad_(True), e, 0, c["N"], fn, c["N"],
-                               routed_experts_fn=routed)
-        o.backward(dout)
-    ms, per = _timed_steps(step_c4, args.warmup, steps)
-    flops = 18.0 * c["T"] * c["K"] * c["H"] * c["I"]
-    wbytes = 3 * 3 * c["N"] * c["H"] * c["I"] * 2
-    with torch.no_grad():
-        _, e = SoftmaxTopkRouterFunction.apply(logits, c["K"], False, torch.bfloat16)
-        counts = torch.bincount(e.flatten(), minlength=c["N"])
-    graph_ms = _graph_replay_ms(step_c4, max(steps, 20))
-    out["C4"] = entry(c["T"], ms, per, flops, wbytes, extra={
-        "graph_replay_ms_per_step": round(graph_ms, 4),
-        "workload": "C4 OLMoE-shape layer under Zipf(1.2) routing, 512 tokens (router on injected logits, "
-                    "permutation, expert GEMMs, combine; fwd+bwd)",
-        "rows_per_expert": {"min": int(counts.min()), "median": int(counts.median()), "max": int(counts.max()),
-                            "experts_with_at_most_8_rows": int((counts <= 8).sum())}})
-    del t, logits, dout
+        def step_c4():
+            for v in t.values():
+                v.grad = None
+            w, e = SoftmaxTopkRouterFunction.apply(logits, c["K"], False, torch.bfloat16)
+            o = expert_computation(t["x"], w.detach().requires_grad_(True), e, 0, c["N"], fn, c["N"],
+                                   routed_experts_fn=routed)
+            o.backward(dout)
+        ms, per = _timed_steps(step_c4, args.warmup, steps)
+        flops = 18.0 * c["T"] * c["K"] * c["H"] * c["I"]
+        wbytes = 3 * 3 * c["N"] * c["H"] * c["I"] * 2
+        with torch.no_grad():
+            _, e = SoftmaxTopkRouterFunction.apply(logits, c["K"], False, torch.bfloat16)
+            counts = torch.bincount(e.flatten(), minlength=c["N"])
+        graph_ms = _graph_replay_ms(step_c4, max(steps, 20))
+        out["C4"] = entry(c["T"], ms, per, flops, wbytes, extra={
+            "graph_replay_ms_per_step": round(graph_ms, 4),
+            "workload": "C4 OLMoE-shape layer under Zipf(1.2) routing, 512 tokens (router on injected logits, "
+                        "permutation, expert GEMMs, combine; fwd+bwd)",
+            "rows_per_expert": {"min": int(counts.min()), "median": int(counts.median()), "max": int(counts.max()),
+                                "experts_with_at_most_8_rows": int((counts <= 8).sum())}})
+        del t, logits, dout
 
     # ---- C5 -----------------------------------------------------------------------------------
-    from optimus.models.deepseek_v3.configuration_deepseek_v3 import DeepseekV3ParallelConfig
-    from optimus.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3ParallelMoE
-    inp = sc.dsv3_inputs()
-    c = inp["cfg"]
-    rank = 2
-    blk = DeepseekV3ParallelMoE(DeepseekV3ParallelConfig(expert_parallelism=8),
-                                ParallelDpPpEpTpMapper(expert_parallelism=8, rank=rank)).to(device).to(torch.bfloat16)
-    with torch.no_grad():
-        blk.gate.weight.copy_(inp["router_w"]); blk.gate.e_score_correction_bias.copy_(inp["bias"])
-        for i, m in enumerate(blk.experts):
-            m.gate_proj.weight.copy_(inp["w_gate"][i]); m.up_proj.weight.copy_(inp["w_up"][i])
-            m.down_proj.weight.copy_(inp["w_down"][i])
-        blk.shared_experts.gate_proj.weight.copy_(inp["ws_gate"]); blk.shared_experts.up_proj.weight.copy_(inp["ws_up"])
-        blk.shared_experts.down_proj.weight.copy_(inp["ws_down"])
-    x = inp["x"].to(device).view(2, c["T"] // 2, c["H"]).requires_grad_(True)
-    dout = inp["dout"].to(device).view_as(x)
-    del inp
+    if only in (None, "C5"):
+        from optimus.models.deepseek_v3.configuration_deepseek_v3 import DeepseekV3ParallelConfig
+        from optimus.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3ParallelMoE
+        inp = sc.dsv3_inputs()
+        c = inp["cfg"]
+        rank = 2
+        blk = DeepseekV3ParallelMoE(DeepseekV3ParallelConfig(expert_parallelism=8),
+                                    ParallelDpPpEpTpMapper(expert_parallelism=8, rank=rank)).to(device).to(torch.bfloat16)
+        with torch.no_grad():
+            blk.gate.weight.copy_(inp["router_w"]); blk.gate.e_score_correction_bias.copy_(inp["bias"])
+            for i, m in enumerate(blk.experts):
+                m.gate_proj.weight.copy_(inp["w_gate"][i]); m.up_proj.weight.copy_(inp["w_up"][i])
+                m.down_proj.weight.copy_(inp["w_down"][i])
+            blk.shared_experts.gate_proj.weight.copy_(inp["ws_gate"]); blk.shared_experts.up_proj.weight.copy_(inp["ws_up"])
+            blk.shared_experts.down_proj.weight.copy_(inp["ws_down"])
+        x = inp["x"].to(device).view(2, c["T"] // 2, c["H"]).requires_grad_(True)
+        dout = inp["dout"].to(device).view_as(x)
+        del inp
 
-    def step_c5():
-        for p in blk.parameters():
-            p.grad = None
-        x.grad = None
-        o = blk(x)
-        o.backward(dout)
-    ms, per = _timed_steps(step_c5, max(2, args.warmup // 2), steps)
-    with torch.no_grad():
-        e, _ = blk.gate(x.detach())
-        local = (e >= rank * c["NR"]) & (e < (rank + 1) * c["NR"])
-        tr = int(local.sum())
-        counts = torch.bincount((e[local] - rank * c["NR"]).flatten(), minlength=c["NR"])
-    flops = 18.0 * (tr + c["T"]) * c["H"] * c["I"]
-    wbytes = 3 * 3 * c["NR"] * c["H"] * c["I"] * 2
-    out["C5"] = entry(c["T"], ms, per, flops, wbytes, extra={
-        "workload": "C5 DeepSeek-V3-style layer, one GPU's share: 8192 tokens, hidden 7168, 32 local of 256 routed "
-                    "experts (ffn 2048) + 1 shared expert, sigmoid group-limited top-8 router; fwd+bwd",
-        "routed_rows_on_this_rank": tr,
-        "rows_per_expert": {"min": int(counts.min()), "median": int(counts.median()), "max": int(counts.max())},
-        "note": "expert_gemm_* and mfma_frac cover the routed and the shared expert's products together; "
-                "weight_stream_* counts the 32 routed experts' matrices only"})
-    del blk, x, dout
-    torch.cuda.empty_cache()
+        def step_c5():
+            for p in blk.parameters():
+                p.grad = None
+            x.grad = None
+            o = blk(x)
+            o.backward(dout)
+        ms, per = _timed_steps(step_c5, max(2, args.warmup // 2), steps)
+        with torch.no_grad():
+            e, _ = blk.gate(x.detach())
+            local = (e >= rank * c["NR"]) & (e < (rank + 1) * c["NR"])
+            tr = int(local.sum())
+            counts = torch.bincount((e[local] - rank * c["NR"]).flatten(), minlength=c["NR"])
+        flops = 18.0 * (tr + c["T"]) * c["H"] * c["I"]
+        wbytes = 3 * 3 * c["NR"] * c["H"] * c["I"] * 2
+        out["C5"] = entry(c["T"], ms, per, flops, wbytes, extra={
+            "workload": "C5 DeepSeek-V3-style layer, one GPU's share: 8192 tokens, hidden 7168, 32 local of 256 routed "
+                        "experts (ffn 2048) + 1 shared expert, sigmoid group-limited top-8 router; fwd+bwd",
+            "routed_rows_on_this_rank": tr,
+            "rows_per_expert": {"min": int(counts.min()), "median": int(counts.median()), "max": int(counts.max())},
+            "note": "expert_gemm_* and mfma_frac cover the routed and the shared expert's products together; "
+                    "weight_stream_* counts the 32 routed experts' matrices only"})
+        del blk, x, dout
+        torch.cuda.empty_cache()
     return out
 
 
@@ -605,6 +608,8 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baselines")
     ap.add_argument("--skip-adamw", action="store_true", help="leave out the AdamW workload")
     ap.add_argument("--skip-other", action="store_true", help="leave out the C1 / C4 / C5 configurations")
+    ap.add_argument("--only-config", choices=("C1", "C4", "C5"),
+                    help="only run this one of the other configurations (for profiling)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run four 1 GiB device copies (calibrates the HBM traffic counters)")
     ap.add_argument("--power-probe", action="store_true",
@@ -635,6 +640,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_probe": {"bytes_per_copy": n, "copies": 4}, "n_gpus": 1}))
+        return
+    if args.only_config:
+        print(json.dumps({"other_configs": bench_other_configs(args, device, False, only=args.only_config),
+                          "n_gpus": 1, "note": "one of the parity-test configurations; not the metric"}))
         return
     moe = bench_moe(args, device)
     out = {

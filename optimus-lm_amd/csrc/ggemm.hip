@@ -985,10 +985,14 @@ int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad f
     return om_launch_status();
 }
 
-// the tile shape launch_rows_auto picks
+// The tile shape launch_rows_auto picks: 256x256 when the extents allow it, the experts hold enough
+// rows to fill such tiles, and there are enough of them for at least half the CUs (a tiny problem is
+// spread over more CUs by the 128x128 tile).
 template <int EPI> bool uses_big_tile(int n_cols, int n_experts, int64_t rows) {
     constexpr int div = (EPI == EPI_SWIGLU) ? 2 : 1;
-    return n_cols % (256 / div) == 0 && rows >= static_cast<int64_t>(n_experts) * 192;
+    if (n_cols % (256 / div) != 0 || rows < static_cast<int64_t>(n_experts) * 192) return false;
+    const int64_t tiles = ((rows + 255) / 256) * (n_cols / (256 / div));
+    return tiles * 2 >= device_cu_count() || n_cols % (128 / div) != 0;
 }
 
 template <int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = false>
@@ -1068,7 +1072,9 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inde
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
     hipStream_t st = om_stream(stream);
-    const bool big = N % 256 == 0 && K % 256 == 0;
+    // 256x256 tiles unless they are too few to occupy half the CUs
+    const bool big = N % 256 == 0 && K % 256 == 0 &&
+                     static_cast<int64_t>(G) * (N / 256) * (K / 256) * 2 >= device_cu_count();
     p.tiles_e = big ? (N / 256) * (K / 256) : (N / 128) * (K / 128);
     const int64_t tiles = static_cast<int64_t>(p.tiles_e) * G;
     if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
