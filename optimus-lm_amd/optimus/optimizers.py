@@ -16,6 +16,28 @@ from optimus.profilers import record_pcl_function
 _STATE_KEYS = ("flat_exp_avg", "flat_exp_avg_sq", "flat_fp32_master_param")
 
 
+_SHARD_STATE_KEYS = ("flat_exp_avg_shard", "flat_exp_avg_sq_shard", "flat_fp32_master_param_shard")
+_ALLREDUCE_PART = 128 * 1024 * 1024      # elements per call of the chunked all-reduce (optimizers.py:11-17)
+
+
+class ProcessGroupExchange:
+    """The three collectives of the sharded step, made through torch.distributed exactly where the
+    reference makes them (optimus/optimizers.py:362-375, :402, :481-494).  Without an initialised
+    process group `active()` is false and the step is the single-process one."""
+
+    def active(self):
+        return torch.distributed.is_available() and torch.distributed.is_initialized()
+
+    def reduce_scatter(self, shard, full, group):
+        torch.distributed.reduce_scatter_tensor(shard, full, group=group)
+
+    def all_reduce(self, tensor, group=None):
+        torch.distributed.all_reduce(tensor, group=group)
+
+    def all_gather(self, full, shard, group):
+        torch.distributed.all_gather_into_tensor(full, shard, group=group)
+
+
 class MixedPrecisionAdamW(Optimizer):
     """AdamW over five flat buffers, interface of the reference class (optimus/optimizers.py:19-225).
 
@@ -24,7 +46,10 @@ class MixedPrecisionAdamW(Optimizer):
     construction each `p.data` and `p.grad` is a view of its slice, so backward accumulates straight
     into the buffer the update kernel reads.  In float32 mode the master weights are `flat_param`
     itself.  Constraints kept from the reference: one parameter group, `device` given, no expert
-    parallelism; beyond it: one GPU (`num_shards == 1`, no tensor parallelism), float32 or bfloat16.
+    parallelism; beyond it: no tensor parallelism, float32 or bfloat16.  With `num_shards > 1` and an
+    initialised process group the gradients are all-reduced over `group` and averaged before the
+    norm, where the reference does it (optimus/optimizers.py:120-133); without a process group the
+    step is the single-process one.
     """
 
     def __init__(self,
@@ -54,9 +79,6 @@ class MixedPrecisionAdamW(Optimizer):
             raise AssertionError("This optimizer does not support expert parallelism.")
         if tensor_parallelism != 1:
             raise AssertionError("tensor parallelism is outside the single-GPU hot path")
-        if num_shards != 1:
-            raise NotImplementedError("num_shards > 1 (data-parallel all-reduce) is not part of "
-                                      "the single-GPU hot path")
         # attributes the training driver and the sharded variants of the reference read
         for name, value in (("model", model), ("warmup_steps", warmup_steps), ("dtype", dtype),
                             ("device", device), ("profiler", profiler), ("group", group),
@@ -71,6 +93,7 @@ class MixedPrecisionAdamW(Optimizer):
             setattr(self, name, value)
         self.step_id = 0
         self.opt_store_clipped_grads = True   # leave flat_grad clipped after step(), as the reference does
+        self.exchange = ProcessGroupExchange()
 
         # layout: one running offset over the group's parameters
         self.param_list = list(self.param_groups[0]["params"])
@@ -144,6 +167,13 @@ class MixedPrecisionAdamW(Optimizer):
         return total.to(self.flat_grad.dtype, copy=True), (coef if clip_now else None)
 
     def step(self, closure=None):
+        with record_pcl_function("3dp-comms-1grad_acc-block"):
+            if self.num_shards > 1 and self.flat_param_size > 0 and self.exchange.active():
+                parts = self.flat_grad.split(_ALLREDUCE_PART) if self.opt_use_chunked_allreduce \
+                    else (self.flat_grad,)
+                for part in parts:
+                    self.exchange.all_reduce(part, self.group)
+                self.flat_grad.div_(self.num_shards)
         with record_pcl_function("4opt-step_grad-clip"):
             grad_norm, clip_coef = self._grad_norm_and_clip()
 
@@ -171,28 +201,6 @@ class MixedPrecisionAdamW(Optimizer):
         for key in _STATE_KEYS:
             getattr(self, key).copy_(opt_state_dict[key].to(self.device))
         self.step_id = opt_state_dict["step_id"]
-
-
-_SHARD_STATE_KEYS = ("flat_exp_avg_shard", "flat_exp_avg_sq_shard", "flat_fp32_master_param_shard")
-_ALLREDUCE_PART = 128 * 1024 * 1024      # elements per call of the chunked all-reduce (optimizers.py:11-17)
-
-
-class ProcessGroupExchange:
-    """The three collectives of the sharded step, made through torch.distributed exactly where the
-    reference makes them (optimus/optimizers.py:362-375, :402, :481-494).  Without an initialised
-    process group `active()` is false and the step is the single-process one."""
-
-    def active(self):
-        return torch.distributed.is_available() and torch.distributed.is_initialized()
-
-    def reduce_scatter(self, shard, full, group):
-        torch.distributed.reduce_scatter_tensor(shard, full, group=group)
-
-    def all_reduce(self, tensor, group=None):
-        torch.distributed.all_reduce(tensor, group=group)
-
-    def all_gather(self, full, shard, group):
-        torch.distributed.all_gather_into_tensor(full, shard, group=group)
 
 
 class ShardedMixedPrecisionAdamW(Optimizer):

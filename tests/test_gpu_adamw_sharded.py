@@ -287,6 +287,46 @@ def test_job_of_several_ranks_vs_oracle(cuda, oracle_lib, world, flags, grad_sca
         assert kinds == {"reduce_scatter", "all_reduce", "all_gather"}
 
 
+@pytest.mark.parametrize("chunked", [False, True])
+def test_unsharded_optimizer_averages_gradients_over_the_ranks(cuda, oracle_lib, chunked):
+    """MixedPrecisionAdamW with num_shards > 1 and a process group (reference optimizers.py:120-133):
+    the whole flat gradient is all-reduced and divided by the number of ranks, then every rank
+    takes the same norm, clip and update; two ranks as threads."""
+    from optimus.optimizers import MixedPrecisionAdamW
+    world = 2
+    job = Rendezvous(world)
+    opts = []
+    for r in range(world):
+        torch.manual_seed(11)
+        net = _Net().to(torch.bfloat16).to(cuda)
+        opt = MixedPrecisionAdamW(net.parameters(), net, lr=HP["lr"], betas=(HP["beta1"], HP["beta2"]),
+                                  eps=HP["eps"], weight_decay=HP["weight_decay"], dtype=torch.bfloat16,
+                                  device=cuda, num_shards=world, shard_id=r,
+                                  opt_use_chunked_allreduce=chunked)
+        opt.exchange = job.member(r)
+        opts.append(opt)
+    n = opts[0].flat_param_size
+    local = [_grad(n, torch.bfloat16, 300 + r, 1.0) for r in range(world)]
+    for r in range(world):
+        opts[r].flat_grad.copy_(local[r])
+    p = bits(opts[0].flat_param).copy(); w = opts[0].flat_fp32_master_param.cpu().numpy().copy()
+    m = np.zeros(n, np.float32); v = np.zeros(n, np.float32)
+    norms = _run_job(opts)
+
+    mean = (local[0].float() + local[1].float()).to(torch.bfloat16).div_(world)
+    g = bits(mean).copy()
+    _, total, coef = oracle_lib.grad_norm_clip(g, opts[0].param_start_inds, opts[0].param_sizes, 1.0)
+    assert coef < 1.0
+    oracle_lib.scale_grads(g, coef)
+    oracle_lib.adamw_step_bf16(p, g, w, m, v, HP["lr"], HP["beta1"], HP["beta2"], HP["eps"], HP["weight_decay"], 1)
+    for r in range(world):
+        assert float(norms[r]) == total
+        assert np.array_equal(bits(opts[r].flat_grad), g)
+        assert np.array_equal(bits(opts[r].flat_param), p)
+        assert np.array_equal(opts[r].flat_fp32_master_param.cpu().numpy().view(np.uint32), w.view(np.uint32))
+        assert opts[r].exchange.calls == ["all_reduce"]
+
+
 def test_state_dict_keys_and_round_trip(cuda):
     _, a = _make(cuda, torch.bfloat16, num_shards=4, shard_id=2)
     a.flat_grad.copy_(_grad(a.flat_buffer_size, torch.bfloat16, 2, 1e-3))
