@@ -14,16 +14,15 @@ from optimus.profilers import record_pcl_function
 
 
 _STATE_KEYS = ("flat_exp_avg", "flat_exp_avg_sq", "flat_fp32_master_param")
-
-
 _SHARD_STATE_KEYS = ("flat_exp_avg_shard", "flat_exp_avg_sq_shard", "flat_fp32_master_param_shard")
 _ALLREDUCE_PART = 128 * 1024 * 1024      # elements per call of the chunked all-reduce (optimizers.py:11-17)
 
 
 class ProcessGroupExchange:
-    """The three collectives of the sharded step, made through torch.distributed exactly where the
-    reference makes them (optimus/optimizers.py:362-375, :402, :481-494).  Without an initialised
-    process group `active()` is false and the step is the single-process one."""
+    """The collectives of the optimizers' steps, made through torch.distributed exactly where the
+    reference makes them (optimus/optimizers.py:120-133 unsharded; :362-375, :402, :481-494 sharded).
+    Without an initialised process group `active()` is false and the step is the single-process
+    one.  Tests replace the optimizer's `exchange` attribute with an in-process stand-in."""
 
     def active(self):
         return torch.distributed.is_available() and torch.distributed.is_initialized()
