@@ -237,7 +237,7 @@ constexpr int WGRAD_EPILOGUE_STEPS = 3;   // a tile's stores take about as long 
 constexpr int WGRAD_BALANCE_MAX_EXPERTS = 4096;
 __device__ __forceinline__ int wgrad_tile_units(int rows, int bk) {
     const int steps = (rows + bk - 1) / bk;
-    return ((steps + 1) & ~1) + WGRAD_EPILOGUE_STEPS;   // the main loop takes its steps in pairs
+    return steps + WGRAD_EPILOGUE_STEPS;
 }
 __device__ __forceinline__ void wgrad_xcd_run(const int32_t *cum, int n_experts, int tiles_e, int bk, int xcd,
                                               int n_xcd, int lane, int &lo, int &hi) {
@@ -322,7 +322,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     int n0 = 0;                                  // first output column (LDS B row 0)
     int c_begin = 0, c_len = 0;                  // contraction range
     int steps_per_phase = 0, total_steps = 0;
-    int loop_steps = 0;   // steps are taken in pairs: total_steps rounded up to even
+    int loop_steps = 0;   // steps the main loop takes (see setup_tile)
     // Tiles that run together on an XCD share operand slices.  Walking the contraction index from
     // 0 in all of them makes them ask L2 for the same lines at the same time, and all wait for the
     // same fill; a small per-tile offset `rot` lets one tile fetch a slice and the sharers hit it.
@@ -428,7 +428,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         c_len = __builtin_amdgcn_readfirstlane(c_len);
         steps_per_phase = (c_len + BK - 1) / BK;
         total_steps = steps_per_phase * p.phases;
-        loop_steps = (total_steps + 1) & ~1;
+        // the loop takes steps in pairs; fwd/dgrad counts are even (kc % 128 == 0), an odd weight-gradient
+        // count ends with a single step
+        loop_steps = (EPI == EPI_WGRAD) ? total_steps : ((total_steps + 1) & ~1);
         rot = (rot_a + rot_b) % (steps_per_phase > 0 ? steps_per_phase : 1);
 #pragma unroll
         for (int i = 0; i < A_LOADS; i++) {
@@ -487,15 +489,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         return true;
     };
 
-    // Loads of contraction step `step` into `stage`.  The padding step of an odd step count (the
-    // loop works on pairs of steps) re-reads the last valid slice; its A tile is zeroed.
+    // Loads of contraction step `step` into `stage`.
     // Loads [lo, hi) of the step's list (A loads first, then B loads); lo and hi are constants
     // after unrolling.
     auto issue_part = [&](int step, char *stage, int lo, int hi) {
         if (step >= loop_steps) return;                    // nothing left to fetch for this tile
         const int ph = (step >= steps_per_phase) ? 1 : 0;  // at most two phases
         const int sp = step - ph * steps_per_phase;
-        int c0 = (sp < steps_per_phase ? rotated(sp) : sp) * BK;   // padding steps stay past the end
+        int c0 = (sp < steps_per_phase ? rotated(sp) : sp) * BK;
         if (EPI != EPI_WGRAD && c0 > c_len - BK) c0 = c_len - BK;
         // first contraction row that this step's STRIDED loads may touch, folded into the scalar base
         // (rows are clamped into the segment, so the base is clamped the same way)
@@ -742,7 +743,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
     // Steps are taken in pairs so the stage names are static; an odd step count (wgrad only: the
-    // host requires kc % 128 == 0 otherwise) is padded with a step whose A tile is all zero.
+    // host requires kc % 128 == 0 otherwise) ends with a single step.
     if (loop_steps > 0) {
         if (!prefetched) issue_loads(0, stage0);
         __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -753,7 +754,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         const int n_steps = loop_steps;
         for (int step = 0; step < n_steps; step += 2) {
             half_step(stage0, stage1, step);
-            half_step(stage1, stage0, step + 1);
+            if (EPI != EPI_WGRAD || step + 1 < n_steps) half_step(stage1, stage0, step + 1);
         }
     }
     __syncthreads();  // the stages are dead: stage 1 becomes the strips, stage 0 the next tile's
