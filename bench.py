@@ -134,6 +134,46 @@ def bench_moe(args, device):
                                      "flops_per_step": 9 * prod_flops, "ms_per_step": round(gemm_ms, 3),
                                      "achieved": round(9 * prod_flops / (gemm_ms * 1e-3) / 1e12, 1),
                                      "frac": round(9 * prod_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}}
+    # The same step the way the reference's trainer runs it: the parameters' gradients are live views
+    # of the optimizer's flat gradient buffer (optimizers.py:105-111) and every backward adds into
+    # them (dist_train.py:154); the weight-gradient GEMMs do that sum in their epilogues.  Timed as
+    # one micro-batch of an accumulation sequence, and with the buffer zeroed before every step.
+    from optimus.optimizers import MixedPrecisionAdamW
+    opt = MixedPrecisionAdamW(blk.parameters(), blk, lr=4e-4, dtype=torch.bfloat16, device=device,
+                              skip_optimizer_step=True)
+
+    def step_accumulating():
+        x.grad = None
+        out, _ = blk(x)
+        out.backward(dout)
+
+    def step_zeroed():
+        opt.zero_grad()
+        step_accumulating()
+
+    def host_timed(fn, n):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / n
+    opt.zero_grad()
+    ms_acc = host_timed(step_accumulating, args.steps)
+    ms_zero = host_timed(step_zeroed, args.steps)
+    _native.launch_log = []
+    step_zeroed()
+    torch.cuda.synchronize()
+    acc_log, _native.launch_log = _native.launch_log, None
+    flat_grad_step = {
+        "what": "the C3 step with every p.grad a live view of MixedPrecisionAdamW.flat_grad: weight gradients are "
+                "added into the buffer by the GEMM epilogues (om_grouped_gemm_wgrad_*_accumulate)",
+        "ms_per_step_accumulating": round(ms_acc, 3), "ms_per_step_with_zero_grad": round(ms_zero, 3),
+        "over_detached_step": round(ms_acc / ms_per_step, 4),
+        "wgrad_launches": sorted({nm for nm, _, _ in acc_log if "wgrad" in nm})}
+    del opt
     # Yardstick, not part of the metric: the vendor library's dense bf16 GEMM (torch.matmul ->
     # hipBLASLt) on the two dense shapes with the same row count, contraction and data as the expert
     # products (one expert's weights for all 131072 rows).  With random operands the chip runs the
@@ -162,7 +202,8 @@ def bench_moe(args, device):
         "frac_of_peak": [round(lib_up / PEAK_BF16_TFLOPS, 4), round(lib_down / PEAK_BF16_TFLOPS, 4)]}
     del blk, x, dout
     torch.cuda.empty_cache()
-    return dict(T=T, ms_per_step=ms_per_step, roofline=roofline, kernels=kernels, cfg=c)
+    return dict(T=T, ms_per_step=ms_per_step, roofline=roofline, kernels=kernels, cfg=c,
+                flat_grad_step=flat_grad_step)
 
 
 def _timed_steps(step, warmup, steps):
@@ -653,7 +694,7 @@ def main():
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "C3 OLMoE-1B-7B-shape MoE layer fwd+bwd: 16384 tokens (4x4096), hidden "
                                "2048, 64 experts, top-8, ffn 1024, fp32 router logits, no dropping"},
-        "roofline": moe["roofline"], "kernels": moe["kernels"],
+        "roofline": moe["roofline"], "kernels": moe["kernels"], "flat_grad_step": moe["flat_grad_step"],
     }
     # GPU workloads first, back to back: the seconds of CPU baseline in between would let the GPU
     # fall into its idle power state right before the HBM-bound measurement

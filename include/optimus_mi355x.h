@@ -502,6 +502,30 @@ int om_moe_row_weights_grad(const float *row_dot, int parts, const int32_t *sele
                             void *routing_weights_grad, int64_t RT, int K, int weights_dtype,
                             void *stream);
 
+/* Weight gradients added to a gradient buffer in place.  In the reference's training set-up every
+ * p.grad is a view of the optimizer's flat gradient buffer (optimus/optimizers.py:105-111) that is
+ * zeroed in place (:117-118), and micro-batches accumulate into it (dist_train.py:154): autograd
+ * ends every weight-gradient GEMM with `p.grad += dW`.  These forms do that sum in the GEMM's
+ * epilogue:  weight_grad = cast(float(weight_grad) + float(cast(dW)))  in the gradient's dtype,
+ * the bits of the in-place add on a freshly rounded dW, without dW being written or re-read.
+ * Arguments as the entry points of the same name without the suffix; weight_grad is read and
+ * written (every element, also those of experts without rows).                               */
+int om_grouped_gemm_wgrad_accumulate(const void *output_grad, const void *input, void *weight_grad,
+                                     const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                                     int64_t w_stride, void *stream);
+int om_grouped_gemm_wgrad_gathered_accumulate(const void *output_grad, const void *input,
+                                              const int32_t *input_rows, int64_t src_rows,
+                                              void *weight_grad, const int32_t *cum_token_counts,
+                                              int64_t rows, int G, int N, int K, int64_t w_stride,
+                                              void *stream);
+int om_grouped_gemm_wgrad_gathered_out_accumulate(const void *output_grad, const int32_t *output_grad_rows,
+                                                  int64_t src_rows, const void *input, void *weight_grad,
+                                                  const int32_t *cum_token_counts, int64_t rows, int G,
+                                                  int N, int K, int64_t w_stride, void *stream);
+int om_grouped_gemm_wgrad_f32_accumulate(const float *output_grad, const float *input, float *weight_grad,
+                                         const int32_t *cum_token_counts, int64_t rows, int G, int N,
+                                         int K, int64_t w_stride, void *stream);
+
 /* Stand-alone SwiGLU glue (moe.py:401-402 forward; moe.py:37-41 and :133-147 backward),
  * for callers that keep the three GEMMs separate.  n elements, dtype OM_F32 or OM_BF16.   */
 int om_swiglu_fwd(const void *g, const void *u, void *h, int64_t n, int dtype, void *stream);

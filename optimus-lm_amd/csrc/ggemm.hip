@@ -88,6 +88,7 @@ struct GemmParams {
     int m_tiles_max;            // fwd/dgrad: upper bound on row tiles
     int total_tiles;            // logical tiles of the launch (the blocks loop over them)
     int tiles_e;                // wgrad: tiles per expert
+    int accumulate;             // wgrad: C[g] = bf16(float(C[g]) + float(bf16(acc))) instead of C[g] = acc
 };
 
 typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_ptr;
@@ -820,9 +821,22 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             wrow_all[(ROWW && EPI == EPI_SWIGLU) ? i : 0] = (m < e_row_end) ? p.row_scale[m] : 0.0f;
         }
     }
+    // Weight gradient added to what the output already holds (a gradient buffer that several
+    // backward passes accumulate into): the old values of a strip are fetched before the strip is
+    // turned around, and the sum is what an in-place bf16 `grad += dW` gives, two roundings.
+    const bool acc_out = EPI == EPI_WGRAD && p.accumulate != 0;
+    u32x4 old_out[EPI == EPI_WGRAD ? ITS : 1];
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int64_t m0 = static_cast<int64_t>(e_row_begin) + wm_e * WM + i * 32;  // first row of the strip
+        if (EPI == EPI_WGRAD && acc_out) {
+#pragma unroll
+            for (int it = 0; it < ITS; it++) {
+                const int q = it * 64 + lane_e;
+                const int64_t o = (m0 + q / CPRW) * p.ldc + col0 + (q % CPRW) * 8;
+                old_out[EPI == EPI_WGRAD ? it : 0] = *reinterpret_cast<const u32x4 *>(Cb + o);
+            }
+        }
         if (EPI == EPI_SWIGLU) {
             const float wrow = wrow_all[(ROWW && EPI == EPI_SWIGLU) ? i : 0];   // ROWW: h = w[row] * silu(g) * u, one rounding
 #pragma unroll
@@ -915,7 +929,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                 const int64_t m = m0 + q / CPRW;
                 if (EPI == EPI_WGRAD || m < e_row_end) {
                     const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
-                    *reinterpret_cast<u32x4 *>(Cb + o) = strip_get(0, q / CPRW, q % CPRW);
+                    u32x4 v = strip_get(0, q / CPRW, q % CPRW);
+                    if (EPI == EPI_WGRAD && acc_out) {
+                        float fresh[8], old[8];
+                        Elem<uint16_t>::unpack(v, fresh);
+                        Elem<uint16_t>::unpack(old_out[EPI == EPI_WGRAD ? it : 0], old);
+#pragma unroll
+                        for (int x = 0; x < 4; x++)
+                            v[x] = pack2_bf16(old[2 * x] + fresh[2 * x], old[2 * x + 1] + fresh[2 * x + 1]);
+                    }
+                    *reinterpret_cast<u32x4 *>(Cb + o) = v;
                     if (EPI == EPI_SWIGLU) {
                         *reinterpret_cast<u32x4 *>(p.C1 + o) = strip_get(1, q / CPRW, q % CPRW);
                         *reinterpret_cast<u32x4 *>(p.C2 + o) = strip_get(2, q / CPRW, q % CPRW);
@@ -1053,7 +1076,7 @@ namespace {
 // [src_rows, N] matrix (the token gather folded into the loads)
 int wgrad_launch(const void *output_grad, const void *input, const int32_t *index, int gather,
                  int64_t src_rows, void *weight_grad, const int32_t *cum_token_counts, int64_t rows, int G,
-                 int N, int K, int64_t w_stride, void *stream) {
+                 int N, int K, int64_t w_stride, void *stream, bool accumulate = false) {
     if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
     // rows == 0 (nothing routed to these experts): the activations may be empty tensors without
     // storage; the launch then only writes zeros
@@ -1072,6 +1095,7 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inde
         !fits_gather(src_rows * (gather == GATHER_WA ? N : K)))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
+    p.accumulate = accumulate ? 1 : 0;
     hipStream_t st = om_stream(stream);
     // 256x256 tiles unless they are too few to occupy half the CUs
     const bool big = N % 256 == 0 && K % 256 == 0 &&
@@ -1124,6 +1148,37 @@ extern "C" int om_grouped_gemm_wgrad_gathered_out(const void *output_grad, const
     if (src_rows < 1) return OM_ERR_SHAPE;
     return wgrad_launch(output_grad, input, output_grad_rows, GATHER_WA, src_rows, weight_grad,
                         cum_token_counts, rows, G, N, K, w_stride, stream);
+}
+
+// The accumulating forms: weight_grad += dW in the gradient's dtype, inside the epilogue.
+extern "C" int om_grouped_gemm_wgrad_accumulate(const void *output_grad, const void *input, void *weight_grad,
+                                                const int32_t *cum_token_counts, int64_t rows, int G, int N,
+                                                int K, int64_t w_stride, void *stream) {
+    return wgrad_launch(output_grad, input, nullptr, GATHER_NONE, 0, weight_grad, cum_token_counts, rows, G,
+                        N, K, w_stride, stream, true);
+}
+
+extern "C" int om_grouped_gemm_wgrad_gathered_accumulate(const void *output_grad, const void *input,
+                                                         const int32_t *input_rows, int64_t src_rows,
+                                                         void *weight_grad, const int32_t *cum_token_counts,
+                                                         int64_t rows, int G, int N, int K, int64_t w_stride,
+                                                         void *stream) {
+    if (!input_rows) return OM_ERR_NULL;
+    if (src_rows < 1) return OM_ERR_SHAPE;
+    return wgrad_launch(output_grad, input, input_rows, GATHER_B, src_rows, weight_grad, cum_token_counts,
+                        rows, G, N, K, w_stride, stream, true);
+}
+
+extern "C" int om_grouped_gemm_wgrad_gathered_out_accumulate(const void *output_grad,
+                                                             const int32_t *output_grad_rows, int64_t src_rows,
+                                                             const void *input, void *weight_grad,
+                                                             const int32_t *cum_token_counts, int64_t rows,
+                                                             int G, int N, int K, int64_t w_stride,
+                                                             void *stream) {
+    if (!output_grad_rows) return OM_ERR_NULL;
+    if (src_rows < 1) return OM_ERR_SHAPE;
+    return wgrad_launch(output_grad, input, output_grad_rows, GATHER_WA, src_rows, weight_grad,
+                        cum_token_counts, rows, G, N, K, w_stride, stream, true);
 }
 
 namespace {

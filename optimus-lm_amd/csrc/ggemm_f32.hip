@@ -27,6 +27,7 @@ struct F32Params {
     const int32_t *cum;
     int64_t lda, ldb, ldc, strideB, strideC;
     int n_experts, n_cols, kc;
+    int accumulate;   // wgrad: C += product instead of C = product
 };
 
 // Fill tile[row][c] (64 x 16) from an operand.  CONTIG: element (row, c) at base[(r0+row)*ld + c0+c],
@@ -53,7 +54,7 @@ template <int AKIND, int BKIND>
 __device__ __forceinline__ void tile_product(const float *A, int64_t lda, int64_t a_r0, int64_t a_rend,
                                              const float *B, int64_t ldb, int64_t b_r0, int64_t b_rend,
                                              int64_t c0, int64_t c1, float *C, int64_t ldc, int64_t m0,
-                                             int64_t m_end, int64_t n0) {
+                                             int64_t m_end, int64_t n0, bool accumulate = false) {
     __shared__ float ta[TB][PITCH], tb[TB][PITCH];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
@@ -79,7 +80,9 @@ __device__ __forceinline__ void tile_product(const float *A, int64_t lda, int64_
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             f4 v = {acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
-            *reinterpret_cast<f4 *>(C + m * ldc + n0 + wn + q * 8 + (lane >> 5) * 4) = v;
+            f4 *dst = reinterpret_cast<f4 *>(C + m * ldc + n0 + wn + q * 8 + (lane >> 5) * 4);
+            if (accumulate) v += *dst;
+            *dst = v;
         }
     }
 }
@@ -116,7 +119,7 @@ __global__ __launch_bounds__(256) void ggemm_f32_wgrad_kernel(const F32Params p)
     const int64_t n0 = static_cast<int64_t>(blockIdx.y) * TB, k0 = static_cast<int64_t>(blockIdx.x) * TB;
     float *C = p.C + expert * p.strideC;
     tile_product<F_STRIDED, F_STRIDED>(p.A, p.lda, n0, n0 + TB, p.B, p.ldb, k0, k0 + TB, r0, r1, C, p.ldc,
-                                       n0, n0 + TB, k0);
+                                       n0, n0 + TB, k0, p.accumulate != 0);
 }
 
 inline bool mult64(int64_t v) { return v > 0 && v % 64 == 0; }
@@ -164,9 +167,10 @@ extern "C" int om_grouped_gemm_dgrad_f32(const float *output_grad, const float *
     return om_launch_status();
 }
 
-extern "C" int om_grouped_gemm_wgrad_f32(const float *output_grad, const float *input, float *weight_grad,
-                                         const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
-                                         int64_t w_stride, void *stream) {
+namespace {
+int wgrad_f32_launch(const float *output_grad, const float *input, float *weight_grad,
+                     const int32_t *cum_token_counts, int64_t rows, int G, int N, int K, int64_t w_stride,
+                     void *stream, bool accumulate) {
     if (rows < 0 || G < 1 || G > 65535 || !mult64(N) || !mult64(K)) return OM_ERR_SHAPE;
     if (!weight_grad || !cum_token_counts || (rows > 0 && (!output_grad || !input))) return OM_ERR_NULL;
     if (!om_aligned16(output_grad) || !om_aligned16(input) || !om_aligned16(weight_grad)) return OM_ERR_ALIGN;
@@ -177,6 +181,23 @@ extern "C" int om_grouped_gemm_wgrad_f32(const float *output_grad, const float *
     if (p.strideC % 4 != 0) return OM_ERR_ALIGN;
     if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideC * G) || N / TB > 65535) return OM_ERR_SHAPE;
     p.n_experts = G; p.n_cols = K; p.kc = N;
+    p.accumulate = accumulate ? 1 : 0;
     ggemm_f32_wgrad_kernel<<<dim3(K / TB, N / TB, G), dim3(256), 0, om_stream(stream)>>>(p);
     return om_launch_status();
+}
+}  // namespace
+
+extern "C" int om_grouped_gemm_wgrad_f32(const float *output_grad, const float *input, float *weight_grad,
+                                         const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
+                                         int64_t w_stride, void *stream) {
+    return wgrad_f32_launch(output_grad, input, weight_grad, cum_token_counts, rows, G, N, K, w_stride, stream,
+                            false);
+}
+
+extern "C" int om_grouped_gemm_wgrad_f32_accumulate(const float *output_grad, const float *input,
+                                                    float *weight_grad, const int32_t *cum_token_counts,
+                                                    int64_t rows, int G, int N, int K, int64_t w_stride,
+                                                    void *stream) {
+    return wgrad_f32_launch(output_grad, input, weight_grad, cum_token_counts, rows, G, N, K, w_stride, stream,
+                            true);
 }

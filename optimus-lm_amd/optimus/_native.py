@@ -107,6 +107,16 @@ SIGNATURES = {
                                                    c_int, c_i64, c_void_p]),
     "om_grouped_gemm_wgrad_gathered": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p,
                                                c_i64, c_int, c_int, c_int, c_i64, c_void_p]),
+    "om_grouped_gemm_wgrad_accumulate": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
+                                                 c_int, c_i64, c_void_p]),
+    "om_grouped_gemm_wgrad_f32_accumulate": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int,
+                                                     c_int, c_int, c_i64, c_void_p]),
+    "om_grouped_gemm_wgrad_gathered_accumulate": (c_int, [c_void_p, c_void_p, c_void_p, c_i64, c_void_p,
+                                                          c_void_p, c_i64, c_int, c_int, c_int, c_i64,
+                                                          c_void_p]),
+    "om_grouped_gemm_wgrad_gathered_out_accumulate": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p,
+                                                              c_void_p, c_i64, c_int, c_int, c_int, c_i64,
+                                                              c_void_p]),
     "om_moe_row_weights": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int,
                                    c_void_p]),
     "om_merged_mlp_gate_up_fwd_weighted": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p,

@@ -35,6 +35,22 @@ def _device_counts(cum_token_counts, device):
     return cum_token_counts.contiguous()
 
 
+_single_segment_cache = {}
+
+
+def single_segment_counts(rows, device):
+    """cum_token_counts of one expert that owns all `rows` rows: the device int32 tensor [0, rows],
+    built once per (rows, device) so that a dense MLP run through the grouped kernels copies nothing
+    from the host per call.  Read-only by contract."""
+    key = (int(rows), str(device))
+    cum = _single_segment_cache.get(key)
+    if cum is None:
+        if len(_single_segment_cache) >= 64:
+            _single_segment_cache.clear()
+        cum = _single_segment_cache[key] = torch.tensor([0, int(rows)], dtype=torch.int32, device=device)
+    return cum
+
+
 def _expert_stride(weight):
     """Elements between consecutive experts of a [G, out, in] weight whose inner two dims are
     dense; 0 for the packed layout."""
@@ -61,10 +77,11 @@ def _gemm_dtype(*tensors):
     return dt
 
 
-def _grouped_gemm(kind, a, b, out, cum, rows, G, N, K, w_stride):
-    """om_grouped_gemm_{fwd,dgrad,wgrad}[_f32] by the operands' dtype."""
+def _grouped_gemm(kind, a, b, out, cum, rows, G, N, K, w_stride, accumulate=False):
+    """om_grouped_gemm_{fwd,dgrad,wgrad}[_f32][_accumulate] by the operands' dtype; `accumulate`
+    (wgrad only) adds the product to `out` in place."""
     suffix = "_f32" if _gemm_dtype(a, b, out) == torch.float32 else ""
-    name = f"om_grouped_gemm_{kind}{suffix}"
+    name = f"om_grouped_gemm_{kind}{suffix}" + ("_accumulate" if accumulate else "")
     _n.check(getattr(_n.lib(), name)(_n.ptr(a), _n.ptr(b), _n.ptr(out), _n.ptr(cum), rows, G, N, K,
                                      w_stride, _n.stream()), name)
 
@@ -310,6 +327,61 @@ def build_token_permutation(selected_experts, expert_start_idx, expert_end_idx):
 
 
 # ----------------------------------------------------------------------------------------------
+# Weight gradients accumulated in place
+# ----------------------------------------------------------------------------------------------
+# The reference trains with every p.grad a view of the optimizer's flat gradient buffer
+# (optimus/optimizers.py:105-111), zeroed in place (:117-118) and accumulated into over the
+# micro-batches of a step (dist_train.py:154), so autograd finishes each weight-gradient GEMM with an
+# elementwise `p.grad += dW` over the whole weight.  When a weight's .grad is such a live view the
+# backward functions below let the GEMM's epilogue do that sum (the *_accumulate entry points: the
+# same bits) and hand autograd None for the weight.  Set to False to always return fresh gradients.
+accumulate_weight_grads_in_place = True
+
+
+def _live_grad(param):
+    """param.grad if the weight-gradient kernels may add into it in place: a leaf parameter whose
+    gradient already exists as a dense view of a larger buffer, same dtype and shape, with no hooks
+    that would have to see the incoming gradient; else None."""
+    if not accumulate_weight_grads_in_place or torch.is_grad_enabled():
+        return None                     # (grad mode is on in backward only under create_graph)
+    if not (isinstance(param, torch.Tensor) and param.is_leaf and param.requires_grad):
+        return None
+    grad = param.grad
+    if grad is None or not grad._is_view() or grad.dtype != param.dtype or grad.shape != param.shape \
+            or not grad.is_cuda or not grad.is_contiguous() or grad.requires_grad:
+        return None
+    if param._backward_hooks or getattr(param, "_post_accumulate_grad_hooks", None):
+        return None
+    return grad
+
+
+def _grad_sink(leaves):
+    """[G, out, in] tensor over the live gradient buffer(s) of an expert weight, or None.  `leaves`
+    is the parameter itself ([G, out, in], or [out, in] for a single MLP) or the list of the G
+    per-expert [out, in] parameters, whose gradients must then lie at one constant pitch inside one
+    buffer (true when they are views of a flat gradient buffer in parameter order)."""
+    if isinstance(leaves, (list, tuple)):
+        grads = [_live_grad(w) for w in leaves]
+        if any(g is None for g in grads):
+            return None
+        try:
+            return _strided_expert_view(grads)
+        except _n.NativeLibraryError:
+            return None
+    grad = _live_grad(leaves)
+    if grad is not None and grad.dim() == 2:
+        grad = grad.unsqueeze(0)
+    return grad
+
+
+def _weight_grad_out(sink, shape, like):
+    """-> (tensor the weight-gradient GEMM writes, its expert pitch argument, accumulate flag)."""
+    if sink is not None:
+        return sink, _expert_stride(sink), True
+    return torch.empty(shape, dtype=like.dtype, device=like.device), 0, False
+
+
+# ----------------------------------------------------------------------------------------------
 # Grouped GEMM functions
 # ----------------------------------------------------------------------------------------------
 class GroupedGemmFunction(torch.autograd.Function):
@@ -339,12 +411,13 @@ class GroupedGemmFunction(torch.autograd.Function):
         num_experts, ofm, ifm = merged_weight.shape
         rows = input.shape[0]
         input_grad = torch.empty_like(input)
-        merged_weight_grad = torch.empty((num_experts, ofm, ifm), dtype=merged_weight.dtype,
-                                         device=merged_weight.device)
+        weight_grad, pitch, acc = _weight_grad_out(_grad_sink(merged_weight), (num_experts, ofm, ifm),
+                                                   merged_weight)
         _grouped_gemm("dgrad", output_grad, merged_weight, input_grad, cum, rows, num_experts, ofm, ifm,
                       _expert_stride(merged_weight))
-        _grouped_gemm("wgrad", output_grad, input, merged_weight_grad, cum, rows, num_experts, ofm, ifm, 0)
-        return input_grad, merged_weight_grad, None, None, None
+        _grouped_gemm("wgrad", output_grad, input, weight_grad, cum, rows, num_experts, ofm, ifm, pitch,
+                      accumulate=acc)
+        return input_grad, (None if acc else weight_grad), None, None, None
 
 
 def _merged_mlp_forward(x, w_gate, w_up, w_down, cum_token_counts, x_rows=None):
@@ -412,33 +485,59 @@ def _merged_mlp_forward_f32(x, w_gate, w_up, w_down, cum_token_counts, x_rows=No
     return y, cum, g, u, h
 
 
-def _merged_mlp_backward_f32(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows=None):
+def _merged_mlp_backward_f32(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows=None,
+                             sinks=(None, None, None)):
     dy = dy.contiguous()
     xs = _gathered_rows(x, x_rows)
     rows, H = dy.shape
     G, I, _ = w_gate.shape
     new = lambda *shape: torch.empty(shape, dtype=x.dtype, device=x.device)
     dh, dg, du, dx, dx2 = new(rows, I), new(rows, I), new(rows, I), new(rows, H), new(rows, H)
-    dw_gate, dw_up, dw_down = new(G, I, H), new(G, I, H), new(G, H, I)
+    (dw_gate, sg, ag), (dw_up, su, au), (dw_down, sd, ad) = (
+        _weight_grad_out(sinks[0], (G, I, H), x), _weight_grad_out(sinks[1], (G, I, H), x),
+        _weight_grad_out(sinks[2], (G, H, I), x))
     with record_pcl_function("1moeblock--7gmlp_bwd"):
-        _grouped_gemm("wgrad", dy, h, dw_down, cum, rows, G, H, I, 0)
+        _grouped_gemm("wgrad", dy, h, dw_down, cum, rows, G, H, I, sd, accumulate=ad)
         _grouped_gemm("dgrad", dy, w_down, dh, cum, rows, G, H, I, _expert_stride(w_down))
         if rows:
             _n.check(_n.lib().om_swiglu_bwd(_n.ptr(dh), _n.ptr(g), _n.ptr(u), _n.ptr(dg), _n.ptr(du), rows * I,
                                             _n.OM_F32, _n.stream()), "om_swiglu_bwd")
-        _grouped_gemm("wgrad", dg, xs, dw_gate, cum, rows, G, I, H, 0)
-        _grouped_gemm("wgrad", du, xs, dw_up, cum, rows, G, I, H, 0)
+        _grouped_gemm("wgrad", dg, xs, dw_gate, cum, rows, G, I, H, sg, accumulate=ag)
+        _grouped_gemm("wgrad", du, xs, dw_up, cum, rows, G, I, H, su, accumulate=au)
         _grouped_gemm("dgrad", dg, w_gate, dx, cum, rows, G, I, H, _expert_stride(w_gate))
         _grouped_gemm("dgrad", du, w_up, dx2, cum, rows, G, I, H, _expert_stride(w_up))
         dx += dx2
-    return dx, dw_gate, dw_up, dw_down
+    return dx, (None if ag else dw_gate), (None if au else dw_up), (None if ad else dw_down)
 
 
-def _merged_mlp_backward(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows=None):
-    """-> (dx, dw_gate [G,I,H], dw_up [G,I,H], dw_down [G,H,I]), all freshly allocated.  With
-    `x_rows` the MLP input was x[x_rows]; dx is then the gradient of that gathered matrix."""
+def _wgrad(output_grad, input, weight_grad, cum, rows, G, N, K, pitch, accumulate, what,
+           input_rows=None, output_grad_rows=None, src_rows=0):
+    """One of the bf16 weight-gradient entry points: plain, with the rows of `input` or of
+    `output_grad` taken through an index, each writing or (accumulate) adding into weight_grad."""
+    lib, st = _n.lib(), _n.stream()
+    tail = "_accumulate" if accumulate else ""
+    if input_rows is not None:
+        name = "om_grouped_gemm_wgrad_gathered" + tail
+        rc = getattr(lib, name)(_n.ptr(output_grad), _n.ptr(input), _n.ptr(input_rows), src_rows,
+                                _n.ptr(weight_grad), _n.ptr(cum), rows, G, N, K, pitch, st)
+    elif output_grad_rows is not None:
+        name = "om_grouped_gemm_wgrad_gathered_out" + tail
+        rc = getattr(lib, name)(_n.ptr(output_grad), _n.ptr(output_grad_rows), src_rows, _n.ptr(input),
+                                _n.ptr(weight_grad), _n.ptr(cum), rows, G, N, K, pitch, st)
+    else:
+        name = "om_grouped_gemm_wgrad" + tail
+        rc = getattr(lib, name)(_n.ptr(output_grad), _n.ptr(input), _n.ptr(weight_grad), _n.ptr(cum), rows,
+                                G, N, K, pitch, st)
+    _n.check(rc, f"{name}({what})")
+
+
+def _merged_mlp_backward(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows=None, sinks=(None, None, None)):
+    """-> (dx, dw_gate [G,I,H], dw_up [G,I,H], dw_down [G,H,I]).  With `x_rows` the MLP input was
+    x[x_rows]; dx is then the gradient of that gathered matrix.  `sinks` (gate, up, down): a weight
+    whose entry is a tensor gets its gradient added into that tensor by the GEMM and None returned;
+    the others get a freshly allocated gradient."""
     if x.dtype == torch.float32:
-        return _merged_mlp_backward_f32(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows)
+        return _merged_mlp_backward_f32(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows, sinks)
     dy = dy.contiguous()
     rows, H = dy.shape
     G, I, _ = w_gate.shape
@@ -447,30 +546,22 @@ def _merged_mlp_backward(dy, x, w_gate, w_up, w_down, cum, g, u, h, x_rows=None)
     dg = torch.empty_like(g)
     du = torch.empty_like(u)
     dx = torch.empty((rows, H), dtype=x.dtype, device=x.device)
-    dw_gate = torch.empty((G, I, H), dtype=x.dtype, device=x.device)
-    dw_up = torch.empty((G, I, H), dtype=x.dtype, device=x.device)
-    dw_down = torch.empty((G, H, I), dtype=x.dtype, device=x.device)
+    (dw_gate, sg, ag), (dw_up, su, au), (dw_down, sd, ad) = (
+        _weight_grad_out(sinks[0], (G, I, H), x), _weight_grad_out(sinks[1], (G, I, H), x),
+        _weight_grad_out(sinks[2], (G, H, I), x))
     with record_pcl_function("1moeblock--7gmlp_bwd"):
-        _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(dy), _n.ptr(h), _n.ptr(dw_down), _n.ptr(cum),
-                                           rows, G, H, I, 0, st), "om_grouped_gemm_wgrad(down)")
+        _wgrad(dy, h, dw_down, cum, rows, G, H, I, sd, ad, "down")
         _n.check(lib.om_merged_mlp_down_dgrad(_n.ptr(dy), _n.ptr(w_down), _n.ptr(g), _n.ptr(u),
                                               _n.ptr(dg), _n.ptr(du), _n.ptr(cum), rows, G, I, H,
                                               _expert_stride(w_down), st), "om_merged_mlp_down_dgrad")
-        if x_rows is not None and rows > 0:
-            for grad, dw, name in ((dg, dw_gate, "gate"), (du, dw_up, "up")):
-                _n.check(lib.om_grouped_gemm_wgrad_gathered(
-                    _n.ptr(grad), _n.ptr(x), _n.ptr(x_rows), x.shape[0], _n.ptr(dw), _n.ptr(cum), rows,
-                    G, I, H, 0, st), f"om_grouped_gemm_wgrad_gathered({name})")
-        else:
-            _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(dg), _n.ptr(x), _n.ptr(dw_gate), _n.ptr(cum),
-                                               rows, G, I, H, 0, st), "om_grouped_gemm_wgrad(gate)")
-            _n.check(lib.om_grouped_gemm_wgrad(_n.ptr(du), _n.ptr(x), _n.ptr(dw_up), _n.ptr(cum),
-                                               rows, G, I, H, 0, st), "om_grouped_gemm_wgrad(up)")
+        gathered = dict(input_rows=x_rows, src_rows=x.shape[0]) if (x_rows is not None and rows > 0) else {}
+        _wgrad(dg, x, dw_gate, cum, rows, G, I, H, sg, ag, "gate", **gathered)
+        _wgrad(du, x, dw_up, cum, rows, G, I, H, su, au, "up", **gathered)
         _n.check(lib.om_merged_mlp_gate_up_dgrad(_n.ptr(dg), _n.ptr(du), _n.ptr(w_gate),
                                                  _n.ptr(w_up), _n.ptr(dx), _n.ptr(cum), rows, G,
                                                  I, H, _expert_stride(w_gate), st),
                  "om_merged_mlp_gate_up_dgrad")
-    return dx, dw_gate, dw_up, dw_down
+    return dx, (None if ag else dw_gate), (None if au else dw_up), (None if ad else dw_down)
 
 
 class MergedMLPFunction(torch.autograd.Function):
@@ -484,14 +575,22 @@ class MergedMLPFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w_gate, w_up, w_down, cum_token_counts):
+        # a single MLP may hand its three [out, in] weights over as they are
+        ctx.leaves = (w_gate, w_up, w_down)
+        ctx.single = w_gate.dim() == 2
+        if ctx.single:
+            w_gate, w_up, w_down = w_gate.unsqueeze(0), w_up.unsqueeze(0), w_down.unsqueeze(0)
         y, cum, g, u, h = _merged_mlp_forward(x, w_gate, w_up, w_down, cum_token_counts)
         ctx.save_for_backward(x, w_gate, w_up, w_down, cum, g, u, h)
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        dx, dw_gate, dw_up, dw_down = _merged_mlp_backward(dy, *ctx.saved_tensors)
-        return dx, dw_gate, dw_up, dw_down, None
+        sinks = tuple(_grad_sink(w) for w in ctx.leaves)
+        dx, *dws = _merged_mlp_backward(dy, *ctx.saved_tensors, sinks=sinks)
+        if ctx.single:
+            dws = [None if dw is None else dw[0] for dw in dws]
+        return (dx, *dws, None)
 
 
 class GatheredMergedMLPFunction(torch.autograd.Function):
@@ -515,13 +614,31 @@ class GatheredMergedMLPFunction(torch.autograd.Function):
     def backward(ctx, dy):
         (hidden_states, input_indices, cum_expert_counts_ep, output_indices, w_gate, w_up, w_down, cum,
          g, u, h) = ctx.saved_tensors
+        sinks = tuple(_grad_sink(w) for w in (w_gate, w_up, w_down))
         dx_rows, dw_gate, dw_up, dw_down = _merged_mlp_backward(dy, hidden_states, w_gate, w_up, w_down,
-                                                                cum, g, u, h, x_rows=input_indices)
+                                                                cum, g, u, h, x_rows=input_indices,
+                                                                sinks=sinks)
         with record_pcl_function("1moeblock--6gmlp_input_prep_bwd"):
             hidden_states_grad = torch.empty_like(hidden_states)
             pcl_xpu_customops.shuffle_sub_matrix_reduce(dx_rows, cum_expert_counts_ep, output_indices,
                                                         hidden_states_grad)
         return hidden_states_grad, None, None, None, dw_gate, dw_up, dw_down, None
+
+
+def _per_expert_leaves(weight_tuple):
+    """(gate, up, down) lists of the per-expert parameters of a (gate_0, up_0, down_0, gate_1, ...)
+    tuple."""
+    N = len(weight_tuple) // 3
+    return tuple([weight_tuple[3 * n + j] for n in range(N)] for j in range(3))
+
+
+def _per_expert_grads(dwg, dwu, dwd, G):
+    """Gradients in the (gate_0, up_0, down_0, gate_1, ...) order of the inputs; None for a
+    projection whose gradient went into its live buffer."""
+    flat = []
+    for n in range(G):
+        flat += [None if dw is None else dw[n] for dw in (dwg, dwu, dwd)]
+    return flat
 
 
 class GroupMLPFunction(torch.autograd.Function):
@@ -532,20 +649,17 @@ class GroupMLPFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, cum_token_counts, use_triton_path, *weight_tuple):
-        N = len(weight_tuple) // 3
-        wg, wu, wd = [_strided_expert_view([weight_tuple[3 * n + j] for n in range(N)])
-                      for j in range(3)]
+        ctx.leaves = _per_expert_leaves(weight_tuple)
+        wg, wu, wd = [_strided_expert_view(ws) for ws in ctx.leaves]
         y, cum, g, u, h = _merged_mlp_forward(input, wg, wu, wd, cum_token_counts)
         ctx.save_for_backward(input, wg, wu, wd, cum, g, u, h)
         return y
 
     @staticmethod
     def backward(ctx, output_grad):
-        dx, dwg, dwu, dwd = _merged_mlp_backward(output_grad, *ctx.saved_tensors)
-        flat = []
-        for n in range(dwg.shape[0]):
-            flat += [dwg[n], dwu[n], dwd[n]]
-        return (dx, None, None, *flat)
+        sinks = tuple(_grad_sink(ws) for ws in ctx.leaves)
+        dx, dwg, dwu, dwd = _merged_mlp_backward(output_grad, *ctx.saved_tensors, sinks=sinks)
+        return (dx, None, None, *_per_expert_grads(dwg, dwu, dwd, len(ctx.leaves[0])))
 
 
 class GatheredGroupMLPFunction(torch.autograd.Function):
@@ -555,9 +669,8 @@ class GatheredGroupMLPFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden_states, input_indices, cum_expert_counts_ep, output_indices, cum_token_counts,
                 *weight_tuple):
-        N = len(weight_tuple) // 3
-        wg, wu, wd = [_strided_expert_view([weight_tuple[3 * n + j] for n in range(N)])
-                      for j in range(3)]
+        ctx.leaves = _per_expert_leaves(weight_tuple)
+        wg, wu, wd = [_strided_expert_view(ws) for ws in ctx.leaves]
         hidden_states = hidden_states.contiguous()
         y, cum, g, u, h = _merged_mlp_forward(hidden_states, wg, wu, wd, cum_token_counts,
                                               x_rows=input_indices)
@@ -569,16 +682,15 @@ class GatheredGroupMLPFunction(torch.autograd.Function):
     def backward(ctx, output_grad):
         (hidden_states, input_indices, cum_expert_counts_ep, output_indices, wg, wu, wd, cum, g, u,
          h) = ctx.saved_tensors
+        sinks = tuple(_grad_sink(ws) for ws in ctx.leaves)
         dx_rows, dwg, dwu, dwd = _merged_mlp_backward(output_grad, hidden_states, wg, wu, wd, cum, g, u, h,
-                                                      x_rows=input_indices)
+                                                      x_rows=input_indices, sinks=sinks)
         with record_pcl_function("1moeblock--6gmlp_input_prep_bwd"):
             hidden_states_grad = torch.empty_like(hidden_states)
             pcl_xpu_customops.shuffle_sub_matrix_reduce(dx_rows, cum_expert_counts_ep, output_indices,
                                                         hidden_states_grad)
-        flat = []
-        for n in range(dwg.shape[0]):
-            flat += [dwg[n], dwu[n], dwd[n]]
-        return (hidden_states_grad, None, None, None, None, *flat)
+        return (hidden_states_grad, None, None, None, None,
+                *_per_expert_grads(dwg, dwu, dwd, len(ctx.leaves[0])))
 
 
 def routed_mlp_kernel_fits(hidden_states, routing_weights, w_gate, w_down):
@@ -636,8 +748,9 @@ def _routed_mlp_forward(hidden_states, routing_weights, input_indices, cum_exper
 
 def _routed_mlp_backward(dfinal, hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
                          output_indices, selected_experts_indices, w_gate, w_up, w_down, cum, g, u, h,
-                         row_weights):
-    """-> (hidden_states_grad, routing_weights_grad, dw_gate, dw_up, dw_down)."""
+                         row_weights, sinks=(None, None, None)):
+    """-> (hidden_states_grad, routing_weights_grad, dw_gate, dw_up, dw_down); `sinks` as in
+    _merged_mlp_backward."""
     dfinal = dfinal.contiguous()
     T, H = hidden_states.shape
     K = routing_weights.shape[1]
@@ -648,9 +761,9 @@ def _routed_mlp_backward(dfinal, hidden_states, routing_weights, input_indices, 
     dg = torch.empty_like(g)
     du = torch.empty_like(u)
     dx_rows = torch.empty((rows, H), dtype=dt, device=dev)
-    dw_gate = torch.empty((G, I, H), dtype=dt, device=dev)
-    dw_up = torch.empty((G, I, H), dtype=dt, device=dev)
-    dw_down = torch.empty((G, H, I), dtype=dt, device=dev)
+    (dw_gate, sg, ag), (dw_up, su, au), (dw_down, sd, ad) = (
+        _weight_grad_out(sinks[0], (G, I, H), hidden_states), _weight_grad_out(sinks[1], (G, I, H), hidden_states),
+        _weight_grad_out(sinks[2], (G, H, I), hidden_states))
     # the kernel writes the entry of every routed (token, k) pair; pairs outside the expert window
     # stay zero
     if rows == routing_weights.numel():
@@ -664,9 +777,8 @@ def _routed_mlp_backward(dfinal, hidden_states, routing_weights, input_indices, 
             if parts < 1:
                 _n.check(parts, "om_merged_mlp_row_dot_parts")
             row_dot = torch.empty((parts, rows), dtype=torch.float32, device=dev)
-            _n.check(lib.om_grouped_gemm_wgrad_gathered_out(
-                _n.ptr(dfinal), _n.ptr(input_indices), T, _n.ptr(h), _n.ptr(dw_down), _n.ptr(cum), rows,
-                G, H, I, 0, st), "om_grouped_gemm_wgrad_gathered_out(down)")
+            _wgrad(dfinal, h, dw_down, cum, rows, G, H, I, sd, ad, "down", output_grad_rows=input_indices,
+                   src_rows=T)
             _n.check(lib.om_merged_mlp_down_dgrad_weighted(
                 _n.ptr(dfinal), _n.ptr(input_indices), T, _n.ptr(w_down), _n.ptr(g), _n.ptr(u),
                 _n.ptr(row_weights), _n.ptr(dg), _n.ptr(du), _n.ptr(row_dot), _n.ptr(cum), rows, G, I, H,
@@ -675,21 +787,23 @@ def _routed_mlp_backward(dfinal, hidden_states, routing_weights, input_indices, 
                 _n.ptr(row_dot), parts, _n.ptr(selected_experts_indices), _n.ptr(input_indices),
                 _n.ptr(output_indices), _n.ptr(routing_weights_grad), rows, K,
                 _n.dtype_code(routing_weights_grad), st), "om_moe_row_weights_grad")
-            for grad, dw, name in ((dg, dw_gate, "gate"), (du, dw_up, "up")):
-                _n.check(lib.om_grouped_gemm_wgrad_gathered(
-                    _n.ptr(grad), _n.ptr(hidden_states), _n.ptr(input_indices), T, _n.ptr(dw), _n.ptr(cum),
-                    rows, G, I, H, 0, st), f"om_grouped_gemm_wgrad_gathered({name})")
+            _wgrad(dg, hidden_states, dw_gate, cum, rows, G, I, H, sg, ag, "gate", input_rows=input_indices,
+                   src_rows=T)
+            _wgrad(du, hidden_states, dw_up, cum, rows, G, I, H, su, au, "up", input_rows=input_indices,
+                   src_rows=T)
             _n.check(lib.om_merged_mlp_gate_up_dgrad(
                 _n.ptr(dg), _n.ptr(du), _n.ptr(w_gate), _n.ptr(w_up), _n.ptr(dx_rows), _n.ptr(cum), rows,
                 G, I, H, _expert_stride(w_gate), st), "om_merged_mlp_gate_up_dgrad")
         else:   # nothing routed to these experts: the weight gradients are zero
-            for dw, n_, k_ in ((dw_down, H, I), (dw_gate, I, H), (dw_up, I, H)):
-                _n.check(lib.om_grouped_gemm_wgrad(None, None, _n.ptr(dw), _n.ptr(cum), 0, G, n_, k_, 0, st),
-                         "om_grouped_gemm_wgrad(empty)")
+            for dw, n_, k_, acc in ((dw_down, H, I, ad), (dw_gate, I, H, ag), (dw_up, I, H, au)):
+                if not acc:     # (a live gradient buffer stays as it is)
+                    _n.check(lib.om_grouped_gemm_wgrad(None, None, _n.ptr(dw), _n.ptr(cum), 0, G, n_, k_, 0, st),
+                             "om_grouped_gemm_wgrad(empty)")
     with record_pcl_function("1moeblock--6gmlp_input_prep_bwd"):
         pcl_xpu_customops.shuffle_sub_matrix_reduce(dx_rows, cum_expert_counts_ep, output_indices,
                                                     hidden_states_grad)
-    return hidden_states_grad, routing_weights_grad, dw_gate, dw_up, dw_down
+    return (hidden_states_grad, routing_weights_grad, None if ag else dw_gate, None if au else dw_up,
+            None if ad else dw_down)
 
 
 class RoutedMLPFunction(torch.autograd.Function):
@@ -715,10 +829,10 @@ class RoutedMLPFunction(torch.autograd.Function):
     def forward(ctx, hidden_states, routing_weights, input_indices, cum_expert_counts_ep, output_indices,
                 selected_experts_indices, cum_token_counts, residual, n_merged, *weights):
         if n_merged:
-            wg, wu, wd = weights
+            wg, wu, wd = ctx.leaves = weights
         else:
-            N = len(weights) // 3
-            wg, wu, wd = [_strided_expert_view([weights[3 * n + j] for n in range(N)]) for j in range(3)]
+            ctx.leaves = _per_expert_leaves(weights)
+            wg, wu, wd = [_strided_expert_view(ws) for ws in ctx.leaves]
         hidden_states = hidden_states.contiguous()
         routing_weights = routing_weights.contiguous()
         if residual is not None:
@@ -735,13 +849,12 @@ class RoutedMLPFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dfinal):
-        dx, drw, dwg, dwu, dwd = _routed_mlp_backward(dfinal, *ctx.saved_tensors)
+        sinks = tuple(_grad_sink(w) for w in ctx.leaves)
+        dx, drw, dwg, dwu, dwd = _routed_mlp_backward(dfinal, *ctx.saved_tensors, sinks=sinks)
         if ctx.n_merged:
             wgrads = (dwg, dwu, dwd)
         else:
-            wgrads = []
-            for n in range(dwg.shape[0]):
-                wgrads += [dwg[n], dwu[n], dwd[n]]
+            wgrads = _per_expert_grads(dwg, dwu, dwd, len(ctx.leaves[0]))
         return (dx, drw, None, None, None, None, None, dfinal if ctx.has_residual else None, None,
                 *wgrads)
 

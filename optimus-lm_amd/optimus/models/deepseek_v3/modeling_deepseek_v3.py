@@ -41,10 +41,9 @@ class DeepseekV3ParallelMLP(nn.Module):
     def forward(self, hidden_states):
         lead = hidden_states.shape[:-1]
         x2 = hidden_states.reshape(-1, hidden_states.shape[-1]).contiguous()
-        cum = torch.tensor([0, x2.shape[0]], dtype=torch.int32, device=x2.device)
-        y = _moe.MergedMLPFunction.apply(x2, self.gate_proj.weight.unsqueeze(0),
-                                         self.up_proj.weight.unsqueeze(0),
-                                         self.down_proj.weight.unsqueeze(0), cum)
+        cum = _moe.single_segment_counts(x2.shape[0], x2.device)
+        y = _moe.MergedMLPFunction.apply(x2, self.gate_proj.weight, self.up_proj.weight,
+                                         self.down_proj.weight, cum)
         return y.reshape(*lead, -1)
 
     def set_parameters_from_full_module(self, module):

@@ -35,10 +35,9 @@ class OlmoeParallelMLP(nn.Module):
         """x [rows, H] -> [rows, H] through the grouped kernels with a single group."""
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
-        cum = torch.tensor([0, x2.shape[0]], dtype=torch.int32, device=x2.device)
-        y = _moe.MergedMLPFunction.apply(x2, self.gate_proj.weight.unsqueeze(0),
-                                         self.up_proj.weight.unsqueeze(0),
-                                         self.down_proj.weight.unsqueeze(0), cum)
+        cum = _moe.single_segment_counts(x2.shape[0], x2.device)
+        y = _moe.MergedMLPFunction.apply(x2, self.gate_proj.weight, self.up_proj.weight,
+                                         self.down_proj.weight, cum)
         return y.reshape(*lead, -1)
 
 
