@@ -6,6 +6,10 @@
 * fast_block_restatement        — optimus/models/common/moe.py:454-621 with the K1..K6
   operators taken from the C restatement of the SYCL kernels (oracle/clib.py) and the expert
   GEMMs as per-expert torch.matmul on slices (moe.py:174-178).
+* fast_block_sequence           — the same block forward AND backward in the tensors' own dtype
+  (bf16 keeps every rounding the reference's sequence of operators has: moe.py:163-215, :396-405,
+  :217-377 and the SYCL kernels behind them); the yardstick for what the reference's own bf16
+  path loses against float32.
 * dense_formula                 — the textbook statement out[t] = sum_k w[t,k] MLP_{e[t,k]}(x[t]),
   evaluated token by token; used on tiny shapes to pin the two loops above.
 
@@ -139,6 +143,99 @@ def fast_block_restatement(hidden_states, routing_weights, selected_experts, w_g
                                          idx["selected_experts_indices"], idx["output_indices"]), dt)
     idx.update(ggemm_input=ggemm_input, g=g, u=u, h=h, ggemm_output=y)
     return final, idx
+
+
+class _SegmentMatmul(torch.autograd.Function):
+    """GroupedGemmFunction with use_triton_path=False (moe.py:163-215): per expert segment
+    out = in @ W[n].T; backward din = dout @ W[n], dW[n] = dout.T @ in.  Every product accumulates in
+    float32 and is rounded once to the operands' dtype, which is what a bf16 GEMM with fp32
+    accumulation (oneDNN on the reference's device, MFMA here) returns."""
+
+    @staticmethod
+    def forward(ctx, inp, weight, cum):
+        out = torch.empty((inp.shape[0], weight.shape[1]), dtype=inp.dtype)
+        for n in range(weight.shape[0]):
+            s, e = int(cum[n]), int(cum[n + 1])
+            out[s:e] = (inp[s:e].float() @ weight[n].float().t()).to(inp.dtype)            # :178
+        ctx.save_for_backward(inp, weight)
+        ctx.cum = cum
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        inp, weight = ctx.saved_tensors
+        cum = ctx.cum
+        din = torch.empty_like(inp)
+        dw = torch.empty_like(weight)
+        for n in range(weight.shape[0]):
+            s, e = int(cum[n]), int(cum[n + 1])
+            din[s:e] = (dout[s:e].float() @ weight[n].float()).to(inp.dtype)               # :208
+            dw[n] = (dout[s:e].float().t() @ inp[s:e].float()).to(weight.dtype)            # :210
+        return din, dw, None
+
+
+class _GatherRows(torch.autograd.Function):
+    """PrepareInputForGroupGemmFunction (moe.py:217-282): index_gather forward,
+    shuffle_sub_matrix_reduce backward (sparse_moe_block.sycl:56-106, :478-532)."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, idx):
+        ctx.idx, ctx.T = idx, hidden_states.shape[0]
+        return _pt(clib.index_gather(_np(hidden_states), idx["input_indices"]), hidden_states.dtype)
+
+    @staticmethod
+    def backward(ctx, grad):
+        idx = ctx.idx
+        return _pt(clib.shuffle_sub_matrix_reduce(_np(grad), idx["cum_expert_counts_ep"],
+                                                  idx["output_indices"], ctx.T), grad.dtype), None
+
+
+class _CombineRows(torch.autograd.Function):
+    """GroupGemmOutputReductionFunction (moe.py:284-377): reduce_ggemm_output forward,
+    reduce_ggemm_output_backward backward (sparse_moe_block.sycl:282-475)."""
+
+    @staticmethod
+    def forward(ctx, y, routing_weights, idx):
+        ctx.idx = idx
+        ctx.save_for_backward(y, routing_weights)
+        return _pt(clib.reduce_ggemm_output(_np(y), _np(routing_weights), idx["cum_expert_counts_ep"],
+                                            idx["selected_experts_indices"], idx["output_indices"]), y.dtype)
+
+    @staticmethod
+    def backward(ctx, dfinal):
+        y, routing_weights = ctx.saved_tensors
+        idx = ctx.idx
+        dy, dw = clib.reduce_ggemm_output_backward(_np(dfinal.contiguous()), _np(y), _np(routing_weights),
+                                                   idx["selected_experts_indices"], idx["input_indices"],
+                                                   idx["output_indices"])
+        return _pt(dy, y.dtype), _pt(dw, routing_weights.dtype), None
+
+
+def fast_block_sequence(hidden_states, routing_weights, selected_experts, w_gate, w_up, w_down, dfinal,
+                        expert_start_idx=0):
+    """expert_computation_block of the fast block (moe.py:473-610), forward and backward, as the
+    reference runs it: K4 gather -> MergedMLP.forward (three GroupedGemmFunction calls, torch's silu
+    and multiply, moe.py:396-405) -> K6 combine, gradients by autograd through exactly those
+    operators.  In bfloat16 every operator rounds its result to bfloat16 as on the reference's
+    device (g, u, silu(g), h, y, dy, dh, d silu, dg, du, the two dx terms and their sum), with
+    fp32 accumulation inside every product and inside K4's and K6's sums.
+
+    All tensors in one dtype (float32 or bfloat16); selected_experts [T,K] int64.
+    Returns (final [T,H], {"x", "routing_weights", "w_gate", "w_up", "w_down"} gradients)."""
+    NR = w_gate.shape[0]
+    idx = clib.index_construction(selected_experts.numpy(), NR, expert_start_idx, expert_start_idx + NR)
+    cum = idx["cum_token_counts"]
+    leaves = {"x": hidden_states, "routing_weights": routing_weights, "w_gate": w_gate, "w_up": w_up,
+              "w_down": w_down}
+    leaves = {k: v.detach().clone().requires_grad_(True) for k, v in leaves.items()}
+    ggemm_input = _GatherRows.apply(leaves["x"], idx)
+    g = _SegmentMatmul.apply(ggemm_input, leaves["w_gate"], cum)            # moe.py:398
+    u = _SegmentMatmul.apply(ggemm_input, leaves["w_up"], cum)              # moe.py:399
+    h = F.silu(g) * u                                                       # moe.py:401-402
+    y = _SegmentMatmul.apply(h, leaves["w_down"], cum)                      # moe.py:404
+    final = _CombineRows.apply(y, leaves["routing_weights"], idx)
+    final.backward(dfinal)
+    return final.detach(), {k: v.grad for k, v in leaves.items()}
 
 
 def rmsnorm(hidden_states, weight, eps, residual=None):

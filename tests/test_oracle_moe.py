@@ -281,3 +281,35 @@ def test_dsv3_block_gradients_match_the_dense_formula():
         assert torch.allclose(a[k].grad, b[k].grad, rtol=1e-4, atol=1e-5), k
     # the routing weights do carry gradient into the router weight
     assert float(a["Wr"].grad.abs().sum()) > 0
+
+
+def test_fast_block_sequence_is_the_layer_and_its_gradients():
+    """fast_block_sequence (gather, three segment products, silu, multiply, combine, and autograd
+    through them) in float32 equals the token-by-token textbook formula and ITS autograd gradients,
+    with and without an expert window; in bfloat16 it is the same function up to bf16 roundings and
+    returns bf16 gradients for every input."""
+    from oracle import moe_layer as L, routing as R
+    torch.manual_seed(5)
+    T, H, N, K, I = 48, 32, 8, 3, 40
+    x = torch.randn(T, H); Wg = torch.randn(N, H) * 0.3
+    wg = torch.randn(N, I, H) * 0.1; wu = torch.randn(N, I, H) * 0.1; wd = torch.randn(N, H, I) * 0.1
+    d = torch.randn(T, H)
+    w, e, _ = R.olmoe_router(x @ Wg.t(), K, False, torch.float32)
+    for start, count in ((0, N), (2, 4)):
+        sl = slice(start, start + count)
+        leaf = {k: v.clone().requires_grad_(True) for k, v in dict(x=x, w=w, wg=wg[sl], wu=wu[sl], wd=wd[sl]).items()}
+        dense = L.dense_formula(leaf["x"], leaf["w"], e, leaf["wg"], leaf["wu"], leaf["wd"], expert_start_idx=start)
+        dense.backward(d)
+        out, grads = L.fast_block_sequence(x, w, e, wg[sl], wu[sl], wd[sl], d, expert_start_idx=start)
+        assert torch.allclose(out, dense, atol=1e-5)
+        for a, b in (("x", "x"), ("routing_weights", "w"), ("w_gate", "wg"), ("w_up", "wu"), ("w_down", "wd")):
+            assert torch.allclose(grads[a], leaf[b].grad, atol=2e-5), a
+    bf = torch.bfloat16
+    out16, g16 = L.fast_block_sequence(x.to(bf), w.to(bf), e, wg.to(bf), wu.to(bf), wd.to(bf), d.to(bf))
+    out32, g32 = L.fast_block_sequence(x.to(bf).float(), w.to(bf).float(), e, wg.to(bf).float(), wu.to(bf).float(),
+                                       wd.to(bf).float(), d.to(bf).float())
+    assert out16.dtype == bf and all(v.dtype == bf for v in g16.values())
+    rel = lambda a, b: float((a.float() - b).abs().mean() / b.abs().mean())
+    assert 1e-3 < rel(out16, out32) < 1e-2                   # rounded, but only rounded
+    for k in g32:
+        assert 1e-3 < rel(g16[k], g32[k]) < 1.5e-2, k
