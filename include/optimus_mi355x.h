@@ -254,7 +254,11 @@ int om_route_sigmoid_topk_bwd(const float *logits, const int64_t *experts, const
  * [expert_start_idx, expert_end_idx).  Results are identical to the reference's:
  *   cum_token_counts [NR+1], cum_expert_counts_ep [T+1], and — for the TR =
  *   cum_token_counts[NR] routed rows — input_indices, output_indices,
- *   selected_experts_indices (each with room for T*K entries; entries >= TR untouched).
+ *   selected_experts_indices (each with room for T*K entries; entries >= TR are set to -1 in
+ *   output_indices and to 0 in the other two, so a caller that sizes the work that follows by
+ *   T*K instead of reading TR back can recognise them: om_moe_row_weights and
+ *   om_moe_row_weights_grad skip them, the expert GEMMs and the per-token sums only ever read
+ *   entries below TR).
  * All outputs stay on the device; nothing is read back.
  * workspace: om_moe_sort_workspace_bytes(T, K, NR) bytes, 4-byte aligned, no pre-zeroing. */
 int64_t om_moe_sort_workspace_bytes(int64_t T, int K, int NR);
@@ -463,7 +467,9 @@ int om_grouped_gemm_wgrad_gathered(const void *output_grad, const void *input,
  * roundings fall in different places (h is rounded after the weight, not before), so results agree
  * with the two-step form to bf16 accuracy, not bit for bit.
  *   om_moe_row_weights       : row_weights[pos] = w[t,k] for every routed entry rt (pos =
- *                              output_indices[rt], t = input_indices[pos], k = sel_idx[rt]); fp32 [RT]
+ *                              output_indices[rt], t = input_indices[pos], k = sel_idx[rt]); fp32 [RT];
+ *                              RT may be an upper bound of the routed entries (T*K) when the index
+ *                              arrays come from om_moe_sort: entries with pos < 0 are skipped
  *   om_merged_mlp_gate_up_fwd_weighted : as ..._gate_up_fwd_gathered, h = bf16(row_weights[r] *
  *                              silu(g) * u) (g and u are stored unweighted)
  *   om_sum_ggemm_output      : final[t,:] = (residual[t,:] +) bf16(sum of the token's rows), no weights;

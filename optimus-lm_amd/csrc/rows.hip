@@ -182,6 +182,7 @@ __global__ __launch_bounds__(256) void row_weights_kernel(
     const int64_t rt = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (rt >= RT) return;
     const int32_t pos = output_indices[rt];
+    if (pos < 0) return;   // past the routed pairs (RT may be an upper bound: see om_moe_sort)
     const int32_t t = input_indices[pos];
     row_weights[pos] = Elem<TW>::load(routing_weights + static_cast<int64_t>(t) * K + selected_experts_indices[rt]);
 }
@@ -195,6 +196,7 @@ __global__ __launch_bounds__(256) void row_weights_grad_kernel(
     const int64_t rt = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (rt >= RT) return;
     const int32_t pos = output_indices[rt];
+    if (pos < 0) return;
     const int32_t t = input_indices[pos];
     float s = 0.0f;
     for (int p0 = 0; p0 < parts; p0 += 8) {

@@ -176,8 +176,17 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(
     int oi_base = hits_base[blockIdx.x];
     for (int w = 0; w < wv; w++) oi_base += wave_hits[w];
     volatile int *off = lds + wv * NR;
+    // Entries past the number of kept pairs (an expert window keeps fewer than T*K) are given fixed
+    // values, so that a caller who sizes its work by T*K instead of reading the count back can tell
+    // them apart: output_indices -1 (no row), the other two 0 (a valid token / slot).
+    const int total_kept = cum_expert_counts_ep[n_pairs / K];
     for (int it = 0; it < SORT_ITERS; it++) {
         const int64_t j = wave_base + it * 64 + lane;
+        if (j < n_pairs && j >= total_kept) {
+            output_indices[j] = -1;
+            input_indices[j] = 0;
+            selected_experts_indices[j] = 0;
+        }
         const int key = local_key(selected_experts, j, n_pairs, start, end, NR);
         const unsigned long long m = match_key(key, nbits);
         const unsigned long long kept = __ballot(key < NR);

@@ -158,7 +158,10 @@ def _gate_backward(x, weight, dlogits, needs, other_grad=None):
 
 
 class GateLogitsFunction(torch.autograd.Function):
-    """fp32 logits of a bf16 gate through om_router_gate_logits (one pass over x)."""
+    """fp32 logits of a bf16 gate through om_router_gate_logits (one pass over x).  Returns
+    (logits, x): the second output is the input itself; a caller that feeds the rest of the layer
+    from it makes that part's input gradient arrive here, where the gate's own input gradient is
+    added to it inside om_router_gate_dgrad instead of by a separate accumulation pass."""
 
     @staticmethod
     def forward(ctx, x, weight):
@@ -179,26 +182,35 @@ class GateLogitsFunction(torch.autograd.Function):
             _n.check(lib.om_router_gate_logits(_n.ptr(x), _n.ptr(weight), T, H, N, _n.ptr(logits),
                                                _n.stream()), "om_router_gate_logits")
         ctx.save_for_backward(x, weight)
-        return logits
+        ctx.set_materialize_grads(False)
+        return logits, x.view_as(x)
 
     @staticmethod
-    def backward(ctx, dlogits):
+    def backward(ctx, dlogits, x_grad):
         x, weight = ctx.saved_tensors
-        return _gate_backward(x, weight, dlogits, ctx.needs_input_grad)
+        if dlogits is None:
+            return x_grad, None
+        return _gate_backward(x, weight, dlogits, ctx.needs_input_grad, other_grad=x_grad)
 
 
-def fp32_logits(x, weight):
-    """Router logits in float32 from 2-D x [T,H] and weight [N,H] (the gate's nn.Linear weight).
+def fp32_logits_with_passthrough(x, weight):
+    """(router logits in float32, x) from 2-D x [T,H] and weight [N,H] (the gate's nn.Linear weight).
     bf16 operands go through the gate kernels (at most 256 experts, H a multiple of 64; anything
-    else raises); a float32 module's gate is torch's own float32 linear."""
+    else raises), and the returned x is GateLogitsFunction's pass-through; a float32 module's gate
+    is torch's own float32 linear and x comes back as it is."""
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         _n.require_cuda_contiguous(x.contiguous(), weight.contiguous())
         _require_gate_shape(weight, 64, "gate projection")
         return GateLogitsFunction.apply(x.contiguous(), weight.contiguous())
     if x.dtype == torch.float32 and weight.dtype == torch.float32:
-        return torch.nn.functional.linear(x, weight)
+        return torch.nn.functional.linear(x, weight), x
     raise TypeError(f"router gate: activations and weight must both be bfloat16 or both float32 "
                     f"(got {x.dtype}, {weight.dtype})")
+
+
+def fp32_logits(x, weight):
+    """Router logits in float32 (see fp32_logits_with_passthrough)."""
+    return fp32_logits_with_passthrough(x, weight)[0]
 
 
 def gate_logits(x, gate):
@@ -748,9 +760,11 @@ def _routed_mlp_forward(hidden_states, routing_weights, input_indices, cum_exper
 
 def _routed_mlp_backward(dfinal, hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
                          output_indices, selected_experts_indices, w_gate, w_up, w_down, cum, g, u, h,
-                         row_weights, sinks=(None, None, None)):
+                         row_weights, sinks=(None, None, None), base=None, rows_is_bound=False):
     """-> (hidden_states_grad, routing_weights_grad, dw_gate, dw_up, dw_down); `sinks` as in
-    _merged_mlp_backward."""
+    _merged_mlp_backward.  `base` [T,H]: another gradient of the same hidden states, added to the
+    result inside the per-token sum (base + cast(sum of the token's rows): autograd's bits).
+    `rows_is_bound`: the index arrays are sized by an upper bound of the routed rows."""
     dfinal = dfinal.contiguous()
     T, H = hidden_states.shape
     K = routing_weights.shape[1]
@@ -766,7 +780,7 @@ def _routed_mlp_backward(dfinal, hidden_states, routing_weights, input_indices, 
         _weight_grad_out(sinks[2], (G, H, I), hidden_states))
     # the kernel writes the entry of every routed (token, k) pair; pairs outside the expert window
     # stay zero
-    if rows == routing_weights.numel():
+    if rows == routing_weights.numel() and not rows_is_bound:
         routing_weights_grad = torch.empty_like(routing_weights)
     else:
         routing_weights_grad = torch.zeros_like(routing_weights)
@@ -800,8 +814,14 @@ def _routed_mlp_backward(dfinal, hidden_states, routing_weights, input_indices, 
                     _n.check(lib.om_grouped_gemm_wgrad(None, None, _n.ptr(dw), _n.ptr(cum), 0, G, n_, k_, 0, st),
                              "om_grouped_gemm_wgrad(empty)")
     with record_pcl_function("1moeblock--6gmlp_input_prep_bwd"):
-        pcl_xpu_customops.shuffle_sub_matrix_reduce(dx_rows, cum_expert_counts_ep, output_indices,
-                                                    hidden_states_grad)
+        if base is None:
+            pcl_xpu_customops.shuffle_sub_matrix_reduce(dx_rows, cum_expert_counts_ep, output_indices,
+                                                        hidden_states_grad)
+        else:
+            _n.require_cuda_contiguous(base)
+            _n.check(lib.om_sum_ggemm_output(
+                _n.ptr(dx_rows), _n.ptr(cum_expert_counts_ep), _n.ptr(output_indices), _n.ptr(base),
+                _n.ptr(hidden_states_grad), T, H, _n.dtype_code(hidden_states_grad), st), "om_sum_ggemm_output")
     return (hidden_states_grad, routing_weights_grad, None if ag else dw_gate, None if au else dw_up,
             None if ad else dw_down)
 
@@ -828,6 +848,10 @@ class RoutedMLPFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden_states, routing_weights, input_indices, cum_expert_counts_ep, output_indices,
                 selected_experts_indices, cum_token_counts, residual, n_merged, *weights):
+        # n_merged: True = merged weights; False = per-expert weights; "bound" forms of both say that
+        # the index arrays are sized by an upper bound of the routed rows (expert_computation)
+        ctx.rows_is_bound = n_merged in ("merged_bound", "per_expert_bound")
+        n_merged = n_merged in (True, "merged_bound")
         if n_merged:
             wg, wu, wd = ctx.leaves = weights
         else:
@@ -850,13 +874,64 @@ class RoutedMLPFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dfinal):
         sinks = tuple(_grad_sink(w) for w in ctx.leaves)
-        dx, drw, dwg, dwu, dwd = _routed_mlp_backward(dfinal, *ctx.saved_tensors, sinks=sinks)
+        dx, drw, dwg, dwu, dwd = _routed_mlp_backward(dfinal, *ctx.saved_tensors, sinks=sinks,
+                                                      rows_is_bound=ctx.rows_is_bound)
         if ctx.n_merged:
             wgrads = (dwg, dwu, dwd)
         else:
             wgrads = _per_expert_grads(dwg, dwu, dwd, len(ctx.leaves[0]))
         return (dx, drw, None, None, None, None, None, dfinal if ctx.has_residual else None, None,
                 *wgrads)
+
+
+class RoutedAndSharedMLPFunction(torch.autograd.Function):
+    """shared_mlp(x) + the routed experts' weighted sum (reference modeling_deepseek_v3.py:265,
+    `self.moe(...) + self.shared_experts(residuals)`) as one function: RoutedMLPFunction over the
+    per-expert weights with the shared MLP's output as its residual.  Same kernels and bits forward
+    as the two functions in sequence.  Backward runs the shared MLP first and hands its input
+    gradient to the routed experts' per-token sum as the base it adds to, so the two input
+    gradients meet inside a kernel (base + cast(sum): what autograd's accumulation gives) and no
+    separate [T,H] addition runs.
+
+    weights: the 3*G routed matrices in GroupMLPFunction's order, then the shared MLP's gate, up,
+    down [out, in] matrices."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, routing_weights, input_indices, cum_expert_counts_ep, output_indices,
+                selected_experts_indices, cum_token_counts, rows_is_bound, *weights):
+        routed, shared = weights[:-3], weights[-3:]
+        ctx.leaves = _per_expert_leaves(routed)
+        ctx.shared_leaves = shared
+        ctx.rows_is_bound = bool(rows_is_bound)
+        wg, wu, wd = [_strided_expert_view(ws) for ws in ctx.leaves]
+        sg, su, sd = [w.unsqueeze(0) for w in shared]
+        hidden_states = hidden_states.contiguous()
+        routing_weights = routing_weights.contiguous()
+        one = single_segment_counts(hidden_states.shape[0], hidden_states.device)
+        y_shared, one, gs, us, hs = _merged_mlp_forward(hidden_states, sg, su, sd, one)
+        final, cum, g, u, h, row_weights = _routed_mlp_forward(
+            hidden_states, routing_weights, input_indices, cum_expert_counts_ep, output_indices,
+            selected_experts_indices, wg, wu, wd, cum_token_counts, y_shared)
+        ctx.save_for_backward(hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                              output_indices, selected_experts_indices, wg, wu, wd, cum, g, u, h,
+                              row_weights, sg, su, sd, one, gs, us, hs)
+        return final
+
+    @staticmethod
+    def backward(ctx, dfinal):
+        saved = ctx.saved_tensors
+        routed_saved, (sg, su, sd, one, gs, us, hs) = saved[:14], saved[14:]
+        hidden_states = saved[0]
+        dfinal = dfinal.contiguous()
+        dx_shared, *dws_shared = _merged_mlp_backward(
+            dfinal, hidden_states, sg, su, sd, one, gs, us, hs,
+            sinks=tuple(_grad_sink(w) for w in ctx.shared_leaves))
+        dx, drw, dwg, dwu, dwd = _routed_mlp_backward(
+            dfinal, *routed_saved, sinks=tuple(_grad_sink(w) for w in ctx.leaves), base=dx_shared,
+            rows_is_bound=ctx.rows_is_bound)
+        dws_shared = [None if dw is None else dw[0] for dw in dws_shared]
+        return (dx, drw, None, None, None, None, None, None,
+                *_per_expert_grads(dwg, dwu, dwd, len(ctx.leaves[0])), *dws_shared)
 
 
 def _strided_expert_view(weights):
@@ -1038,7 +1113,7 @@ class MergedMLP(nn.Module):
 
 def expert_computation(hidden_states, routing_weights, selected_experts, expert_start_idx,
                        expert_end_idx, experts_fn, num_total_experts, gathered_experts_fn=None,
-                       residual=None, routed_experts_fn=None):
+                       residual=None, routed_experts_fn=None, sync_free_window=False):
     """K1..K6 for 2-D hidden_states [T,H]: permute, run `experts_fn(ggemm_input, cum_token_counts)`,
     combine.  Shared by the OLMoE and DeepSeek-V3 blocks.  With `gathered_experts_fn(hidden_states,
     input_indices, cum_expert_counts_ep, output_indices, cum_token_counts)` the experts read the
@@ -1046,13 +1121,28 @@ def expert_computation(hidden_states, routing_weights, selected_experts, expert_
     is residual + combine(...), added inside the combine kernel.  `routed_experts_fn(hidden_states,
     routing_weights, input_indices, cum_expert_counts_ep, output_indices, selected_experts_indices,
     cum_token_counts, residual)` may do gather, experts and combine in one function
-    (RoutedMLPFunction); it returns None when its kernels do not take the operands."""
+    (RoutedMLPFunction); it returns None when its kernels do not take the operands.
+
+    Under an expert window the number of routed rows is only known on the device.  By default it is
+    read back once, like the reference does (moe.py:520).  With `sync_free_window` and a
+    `routed_experts_fn` nothing is read back: the index arrays keep their T*K entries (om_moe_sort
+    marks the unused tail), the activations of the expert MLP are allocated for T*K rows, of which
+    only the routed ones are computed, and the function is called with `rows_is_bound=True`.  That
+    makes the step capturable in a HIP graph at the price of expert_parallelism times the
+    activation memory."""
     T, K = selected_experts.shape
     with record_pcl_function("1moeblock--3index_calculation"):
         (cum_token_counts, cum_expert_counts_ep, input_indices, output_indices,
          selected_experts_indices) = build_token_permutation(selected_experts, expert_start_idx,
                                                              expert_end_idx)
-    if expert_start_idx == 0 and expert_end_idx == num_total_experts:
+    windowed = not (expert_start_idx == 0 and expert_end_idx == num_total_experts)
+    if windowed and sync_free_window and routed_experts_fn is not None:
+        final = routed_experts_fn(hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                                  output_indices, selected_experts_indices, cum_token_counts, residual,
+                                  rows_is_bound=True)
+        if final is not None:
+            return final
+    if not windowed:
         num_routed_tokens = T * K            # every pair is local: no host read
     else:
         num_routed_tokens = int(cum_token_counts[-1].item())   # same host read as moe.py:520
@@ -1120,6 +1210,8 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
         # the routing weight is applied inside the expert MLP and the combine's backward is folded
         # into the down projection's backward GEMMs (RoutedMLPFunction); needs fuse_input_gather
         self.fuse_routing_weights = bool(getattr(config, "fuse_routing_weights", True))
+        # under an expert window: never read the routed row count back (see expert_computation)
+        self.sync_free_expert_window = bool(getattr(config, "sync_free_expert_window", False))
 
     def _experts_fn(self, ggemm_input, cum_token_counts):
         if isinstance(self.experts, MergedMLP):
@@ -1143,7 +1235,8 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
                                               output_indices, cum_token_counts, *mlp_params)
 
     def _routed_experts_fn(self, hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
-                           output_indices, selected_experts_indices, cum_token_counts, residual):
+                           output_indices, selected_experts_indices, cum_token_counts, residual,
+                           rows_is_bound=False):
         if isinstance(self.experts, MergedMLP):
             weights = (self.experts.gate_proj_merged_weight, self.experts.up_proj_merged_weight,
                        self.experts.down_proj_merged_weight)
@@ -1151,7 +1244,8 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
                 return None
             return RoutedMLPFunction.apply(hidden_states, routing_weights, input_indices,
                                            cum_expert_counts_ep, output_indices, selected_experts_indices,
-                                           cum_token_counts, residual, True, *weights)
+                                           cum_token_counts, residual,
+                                           "merged_bound" if rows_is_bound else True, *weights)
         pack_expert_weights(self.experts)
         w0, d0 = self.experts[0].gate_proj.weight, self.experts[0].down_proj.weight
         if not routed_mlp_kernel_fits(hidden_states, routing_weights, w0.unsqueeze(0), d0.unsqueeze(0)):
@@ -1161,7 +1255,7 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
             mlp_params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
         return RoutedMLPFunction.apply(hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
                                        output_indices, selected_experts_indices, cum_token_counts,
-                                       residual, False, *mlp_params)
+                                       residual, "per_expert_bound" if rows_is_bound else False, *mlp_params)
 
     def forward_with_residual(self, hidden_states, residual):
         """(residual + forward(hidden_states)[0], router_logits): the decoder layer's
@@ -1196,7 +1290,8 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
                                      self.expert_start_idx, self.expert_end_idx, self._experts_fn,
                                      self.num_experts, gathered_experts_fn=gathered,
                                      residual=None if residual is None else residual.reshape(-1, h),
-                                     routed_experts_fn=routed)
+                                     routed_experts_fn=routed,
+                                     sync_free_window=self.sync_free_expert_window)
             return out.reshape(b, s, h)
 
         args = [hidden_states, selected_experts, routing_weights]

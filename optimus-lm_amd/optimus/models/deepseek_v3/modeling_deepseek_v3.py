@@ -103,13 +103,19 @@ class DeepseekV3ParallelTopkRouter(nn.Module):
             raise NotImplementedError("force_uniform_routing is not part of this build")
 
     def forward(self, hidden_states):
+        return self.forward_with_passthrough(hidden_states)[:2]
+
+    def forward_with_passthrough(self, hidden_states):
+        """(topk_indices, topk_weights, hidden_states [T,H]): the third result is the gate
+        projection's pass-through of its input; experts fed from it get their input gradient added
+        to the gate's inside the gate's input-gradient kernel (GateLogitsFunction)."""
         hidden_states = hidden_states.reshape(-1, self.config.hidden_size)
-        router_logits = _moe.fp32_logits(hidden_states, self.weight)
+        router_logits, hidden_states = _moe.fp32_logits_with_passthrough(hidden_states, self.weight)
         topk_indices, topk_weights = SigmoidGroupTopkRouterFunction.apply(
             router_logits.contiguous(), self.e_score_correction_bias.float().contiguous(),
             self.n_group, self.topk_group, self.top_k, self.norm_topk_prob,
             self.routed_scaling_factor)
-        return topk_indices, topk_weights
+        return topk_indices, topk_weights, hidden_states
 
 
 class DeepseekV3ParallelMoE(nn.Module):
@@ -148,36 +154,61 @@ class DeepseekV3ParallelMoE(nn.Module):
         return _moe.GatheredGroupMLPFunction.apply(hidden_states, input_indices, cum_expert_counts_ep,
                                                    output_indices, cum_token_counts, *params)
 
-    def _routed_experts_fn(self, hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
-                           output_indices, selected_experts_indices, cum_token_counts, residual):
-        _moe.pack_expert_weights(self.experts)
+    def _routed_kernels_fit(self, hidden_states, routing_weights):
         w0, d0 = self.experts[0].gate_proj.weight, self.experts[0].down_proj.weight
-        if not _moe.routed_mlp_kernel_fits(hidden_states, routing_weights, w0.unsqueeze(0), d0.unsqueeze(0)):
+        return _moe.routed_mlp_kernel_fits(hidden_states, routing_weights, w0.unsqueeze(0), d0.unsqueeze(0))
+
+    def _routed_experts_fn(self, hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
+                           output_indices, selected_experts_indices, cum_token_counts, residual,
+                           rows_is_bound=False, with_shared=False):
+        _moe.pack_expert_weights(self.experts)
+        if not self._routed_kernels_fit(hidden_states, routing_weights):
             return None
         params = []
         for expert in self.experts:
             params += [expert.gate_proj.weight, expert.up_proj.weight, expert.down_proj.weight]
+        if with_shared:
+            sh = self.shared_experts
+            return _moe.RoutedAndSharedMLPFunction.apply(
+                hidden_states, routing_weights, input_indices, cum_expert_counts_ep, output_indices,
+                selected_experts_indices, cum_token_counts, rows_is_bound, *params, sh.gate_proj.weight,
+                sh.up_proj.weight, sh.down_proj.weight)
         return _moe.RoutedMLPFunction.apply(hidden_states, routing_weights, input_indices,
                                             cum_expert_counts_ep, output_indices, selected_experts_indices,
-                                            cum_token_counts, residual, False, *params)
+                                            cum_token_counts, residual,
+                                            "per_expert_bound" if rows_is_bound else False, *params)
 
-    def moe(self, hidden_states, topk_indices, topk_weights, residual=None):
+    def _fuses_routing_weights(self):
+        return getattr(self.config, "fuse_input_gather", True) and \
+            getattr(self.config, "fuse_routing_weights", True)
+
+    def moe(self, hidden_states, topk_indices, topk_weights, residual=None, with_shared=False):
         """Routed part for [T,H] hidden_states (reference :221-244): fp32 weights, fp32 sum over a
         token's local experts, one rounding to the activation dtype.  The local experts read their
         tokens through the permutation index (no gathered copy of the activations) and apply the
         routing weight themselves (RoutedMLPFunction) unless the config switches that off.
-        `residual` [T,H] is added to the rounded result inside the combine kernel."""
-        fuse_gather = getattr(self.config, "fuse_input_gather", True)
-        gathered = self._gathered_experts_fn if fuse_gather else None
-        routed = self._routed_experts_fn if (
-            fuse_gather and getattr(self.config, "fuse_routing_weights", True)) else None
+        `residual` [T,H] is added to the rounded result inside the combine kernel.  `with_shared`
+        (needs the fused path): the shared experts run inside the same function and their output
+        is that residual (RoutedAndSharedMLPFunction)."""
+        gathered = self._gathered_experts_fn if getattr(self.config, "fuse_input_gather", True) else None
+        routed = None
+        if self._fuses_routing_weights():
+            routed = self._routed_experts_fn
+            if with_shared:
+                routed = lambda *a, **kw: self._routed_experts_fn(*a, with_shared=True, **kw)
+        elif with_shared:
+            raise ValueError("with_shared needs the fused routing-weight path")
         return _moe.expert_computation(hidden_states, topk_weights, topk_indices,
                                        self.expert_start_idx, self.expert_end_idx, self._experts_fn,
                                        self.config.n_routed_experts, gathered_experts_fn=gathered,
-                                       residual=residual, routed_experts_fn=routed)
+                                       residual=residual, routed_experts_fn=routed,
+                                       sync_free_window=getattr(self.config, "sync_free_expert_window", False))
 
     def forward(self, hidden_states):
-        topk_indices, topk_weights = self.gate(hidden_states)
+        # the experts are fed from the gate projection's pass-through of the hidden states, so that
+        # their input gradient and the gate's are added inside one kernel
+        topk_indices, topk_weights, flat = self.gate.forward_with_passthrough(hidden_states)
+        hidden_states = flat.view(hidden_states.shape)
 
         def expert_computation_block(hidden_states, topk_indices, topk_weights):
             residuals = hidden_states
@@ -186,6 +217,8 @@ class DeepseekV3ParallelMoE(nn.Module):
             # routed + shared (reference :265): the shared experts' output goes into the combine
             # kernel as its residual, which rounds the routed sum first and then adds: the same two
             # roundings as `moe(...) + shared_experts(...)`
+            if self._fuses_routing_weights() and self._routed_kernels_fit(flat, topk_weights):
+                return self.moe(flat, topk_indices, topk_weights, with_shared=True).view(*orig_shape)
             shared = self.shared_experts(residuals).reshape(flat.shape)
             return self.moe(flat, topk_indices, topk_weights, residual=shared).view(*orig_shape)
 
