@@ -30,20 +30,33 @@ sys.path.insert(0, os.path.join(ROOT, "optimus-lm_amd"))
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM bytes per launch (read + write) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same
-# command, scaled by what the counters read for a plain 1 GiB copy (x2.000 and x1.000); the table
-# and the commands are in profiles/hbm_traffic_c3_expert_gemms_and_c2_adamw.md.  Offline figures:
-# counters cannot be collected inside the timed run.
+# HBM bytes per launch (read + write) come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# same command, scaled by what the counters read for a plain 1 GiB copy: counters cannot be collected
+# inside the timed run, so the figures are kept in a data file next to the kernels, together with the
+# command and the digest of the kernel source they were measured on.  A figure whose source has
+# changed since is not reported (traffic: null).
 MIB = float(1 << 20)
-MEASURED_TRAFFIC_BYTES = {
-    "om_merged_mlp_gate_up_fwd_weighted": (3317 + 768.6) * MIB, "om_grouped_gemm_fwd": (1396.5 + 512) * MIB,
-    "om_merged_mlp_gate_up_dgrad": (3490 + 512) * MIB, "om_merged_mlp_down_dgrad_weighted": (1944.8 + 523.6) * MIB,
-    "om_grouped_gemm_wgrad_gathered": (962.5 + 256) * MIB, "om_grouped_gemm_wgrad_gathered_out": (911.7 + 256) * MIB,
-    "om_adamw_step": (92125 + 92125) * MIB,
-    # entry points a C3 step no longer launches, as measured when it did
-    "om_merged_mlp_gate_up_fwd": (3220 + 768) * MIB, "om_grouped_gemm_wgrad": (927 + 256) * MIB,
-    "om_merged_mlp_down_dgrad": (1952 + 512) * MIB, "om_merged_mlp_gate_up_fwd_gathered": (3288 + 768) * MIB,
-}
+TRAFFIC_FILE = os.path.join(ROOT, "optimus-lm_amd", "csrc", "hbm_traffic_measured.json")
+
+
+def source_digest(name):
+    import hashlib
+    with open(os.path.join(ROOT, "optimus-lm_amd", "csrc", name), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def measured_traffic_bytes(entry):
+    """Measured HBM bytes per launch of a C-ABI entry point, or None when there is no figure for
+    the kernel source as it is now."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None
+    rec = table.get("entries", {}).get(entry)
+    if rec is None or table.get("source_digest", {}).get(rec["source"]) != source_digest(rec["source"]):
+        return None
+    return (rec["fetch_mib"] + rec["write_mib"]) * MIB
 
 GEMM_ENTRY_PRODUCTS = {     # C-ABI entry -> number of [rows x N x K] products per launch
     "om_merged_mlp_gate_up_fwd": 2, "om_grouped_gemm_fwd": 1, "om_grouped_gemm_wgrad": 1,
@@ -51,6 +64,8 @@ GEMM_ENTRY_PRODUCTS = {     # C-ABI entry -> number of [rows x N x K] products p
     "om_merged_mlp_gate_up_fwd_weighted": 2, "om_grouped_gemm_wgrad_gathered_out": 1,
     "om_merged_mlp_down_dgrad_weighted": 1,
     "om_merged_mlp_down_dgrad": 1, "om_merged_mlp_gate_up_dgrad": 2, "om_grouped_gemm_dgrad": 1,
+    "om_grouped_gemm_wgrad_accumulate": 1, "om_grouped_gemm_wgrad_gathered_accumulate": 1,
+    "om_grouped_gemm_wgrad_gathered_out_accumulate": 1,
 }
 
 
@@ -129,7 +144,7 @@ def bench_moe(args, device):
     achieved = GEMM_ENTRY_PRODUCTS[dom] * prod_flops / dom_avg_s / 1e12
     roofline = {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1),
                 "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+                "traffic": measured_traffic_bytes(dom),
                 "all_expert_gemms": {"from": "untimed profiling pass with every entry point bracketed by events",
                                      "flops_per_step": 9 * prod_flops, "ms_per_step": round(gemm_ms, 3),
                                      "achieved": round(9 * prod_flops / (gemm_ms * 1e-3) / 1e12, 1),
@@ -272,15 +287,27 @@ def bench_other_configs(args, device, with_cpu, only=None):
     def gemm_ms(per):
         return sum(v for k, v in per.items() if k in GEMM_ENTRY_PRODUCTS)
 
-    def entry(T, ms, per, flops, weight_bytes=None, extra=None):
+    def entry(T, ms, per, flops, weight_bytes=None, extra=None, bound="mfma"):
         g = gemm_ms(per)
+        tflops = flops / (g * 1e-3) / 1e12
         e = {"ms_per_step": round(ms, 4), "tokens_per_s": round(T / (ms * 1e-3), 1),
              "expert_gemm_ms": round(g, 4), "expert_gemm_flops": flops,
-             "mfma_frac": round(flops / (g * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+             "mfma_frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
         if weight_bytes is not None:
             e["weight_stream_gb_per_s"] = round(weight_bytes / (g * 1e-3) / 1e9, 1)
             e["weight_stream_hbm_frac"] = round(weight_bytes / (g * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
             e["weight_bytes_per_step"] = weight_bytes
+        # the configuration's own roofline object, over all its expert-GEMM launches
+        if bound == "hbm":
+            gbs = weight_bytes / (g * 1e-3) / 1e9
+            e["roofline"] = {"bound": "hbm", "kernel": "all expert GEMM launches of the step (weight streaming)",
+                             "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+        else:
+            e["roofline"] = {"bound": "mfma", "kernel": "all expert GEMM launches of the step",
+                             "achieved": round(tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                             "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}
+        e["expert_gemm_launches_ms"] = {k: round(v, 4) for k, v in sorted(per.items()) if k in GEMM_ENTRY_PRODUCTS}
         if extra:
             e.update(extra)
         return e
@@ -351,7 +378,14 @@ def bench_other_configs(args, device, with_cpu, only=None):
             _, e = SoftmaxTopkRouterFunction.apply(logits, c["K"], False, torch.bfloat16)
             counts = torch.bincount(e.flatten(), minlength=c["N"])
         graph_ms = _graph_replay_ms(step_c4, max(steps, 20))
-        out["C4"] = entry(c["T"], ms, per, flops, wbytes, extra={
+        one_pass = 3 * c["N"] * c["H"] * c["I"] * 2      # every expert's three matrices once
+        per_launch = {   # weight bytes each entry point streams (reads, or writes for the weight gradients)
+            "om_merged_mlp_gate_up_fwd_weighted": one_pass * 2 / 3, "om_grouped_gemm_fwd": one_pass / 3,
+            "om_merged_mlp_down_dgrad_weighted": one_pass / 3, "om_merged_mlp_gate_up_dgrad": one_pass * 2 / 3,
+            "om_grouped_gemm_wgrad_gathered": one_pass * 2 / 3, "om_grouped_gemm_wgrad_gathered_out": one_pass / 3}
+        out["C4"] = entry(c["T"], ms, per, flops, wbytes, bound="hbm", extra={
+            "weight_stream_gb_per_s_by_entry_point": {
+                k: round(b / (per[k] * 1e-3) / 1e9, 1) for k, b in per_launch.items() if k in per},
             "graph_replay_ms_per_step": round(graph_ms, 4),
             "workload": "C4 OLMoE-shape layer under Zipf(1.2) routing, 512 tokens (router on injected logits, "
                         "permutation, expert GEMMs, combine; fwd+bwd)",
@@ -366,8 +400,8 @@ def bench_other_configs(args, device, with_cpu, only=None):
         inp = sc.dsv3_inputs()
         c = inp["cfg"]
         rank = 2
-        blk = DeepseekV3ParallelMoE(DeepseekV3ParallelConfig(expert_parallelism=8),
-                                    ParallelDpPpEpTpMapper(expert_parallelism=8, rank=rank)).to(device).to(torch.bfloat16)
+        c5cfg = DeepseekV3ParallelConfig(expert_parallelism=8)
+        blk = DeepseekV3ParallelMoE(c5cfg, ParallelDpPpEpTpMapper(expert_parallelism=8, rank=rank)).to(device).to(torch.bfloat16)
         with torch.no_grad():
             blk.gate.weight.copy_(inp["router_w"]); blk.gate.e_score_correction_bias.copy_(inp["bias"])
             for i, m in enumerate(blk.experts):
@@ -386,6 +420,12 @@ def bench_other_configs(args, device, with_cpu, only=None):
             o = blk(x)
             o.backward(dout)
         ms, per = _timed_steps(step_c5, max(2, args.warmup // 2), steps)
+        # the same step with the routed-row count left on the device (nothing read back; the expert
+        # activations are allocated for T*K rows): eager, and replayed from a HIP graph
+        c5cfg.sync_free_expert_window = True
+        ms_free, _ = _timed_steps(step_c5, 2, steps)
+        graph_ms = _graph_replay_ms(step_c5, max(steps, 10))
+        c5cfg.sync_free_expert_window = False
         with torch.no_grad():
             e, _ = blk.gate(x.detach())
             local = (e >= rank * c["NR"]) & (e < (rank + 1) * c["NR"])
@@ -396,6 +436,7 @@ def bench_other_configs(args, device, with_cpu, only=None):
         out["C5"] = entry(c["T"], ms, per, flops, wbytes, extra={
             "workload": "C5 DeepSeek-V3-style layer, one GPU's share: 8192 tokens, hidden 7168, 32 local of 256 routed "
                         "experts (ffn 2048) + 1 shared expert, sigmoid group-limited top-8 router; fwd+bwd",
+            "sync_free_window_ms_per_step": round(ms_free, 4), "graph_replay_ms_per_step": round(graph_ms, 4),
             "routed_rows_on_this_rank": tr,
             "rows_per_expert": {"min": int(counts.min()), "median": int(counts.median()), "max": int(counts.max())},
             "note": "expert_gemm_* and mfma_frac cover the routed and the shared expert's products together; "
@@ -606,7 +647,7 @@ def bench_adamw(args, device):
                                    "param/grad + fp32 master/m/v, step 100"},
             "roofline": {"bound": "hbm", "kernel": "om_adamw_step", "achieved": round(gbs, 1),
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
-                         "traffic": MEASURED_TRAFFIC_BYTES["om_adamw_step"], "bytes_per_param": 28, "kernel_avg_ms": round(avg_s * 1e3, 3),
+                         "traffic": measured_traffic_bytes("om_adamw_step"), "bytes_per_param": 28, "kernel_avg_ms": round(avg_s * 1e3, 3),
                          "streaming_ceiling": {
                              "what": "om_adamw_traffic_probe: the update kernel's loads and stores (14 B read + "
                                      "14 B written per parameter, same block shape and cache hints) without "
@@ -712,3 +753,7 @@ def main():
 
 if __name__ == "__main__":
     main()
+    # leave promptly: the line is out, the device memory goes back with the process
+    sys.stdout.flush()
+    sys.stderr.flush()
+    os._exit(0)
