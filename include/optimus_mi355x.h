@@ -57,7 +57,8 @@ const char *om_strerror(int code);
  * param_dtype OM_F32 : grad fp32 and `master` IS the parameter buffer; `param` is ignored
  *                      (the reference aliases them, optimizers.py:100-102).
  * `step` is t = step_id + 1 (1-based).  All five buffers must be 16-byte aligned.
- * n may exceed 2^31.                                                                    */
+ * n may exceed 2^31; beyond 2^33 elements the call makes several launches over consecutive
+ * sub-ranges (element-wise work: the same bits).                                           */
 int om_adamw_step(void *param, const void *grad, float *master, float *exp_avg,
                   float *exp_avg_sq, int64_t n, double lr, double beta1, double beta2,
                   double eps, double weight_decay, int64_t step, int param_dtype,
@@ -277,7 +278,10 @@ int om_moe_sort(const void *selected_experts, int index_dtype, int64_t T, int K,
  * return OM_ERR_WORKSPACE (4 MiB serves e.g. 8M pairs over 256 local experts).  Same results as
  * om_moe_sort, bit for bit.  The array is shared by every call on a GPU: calls that overlap on one
  * GPU (two streams, two threads) race; calls on one stream are ordered and safe.  Nothing in the
- * array needs to start at zero.                                                             */
+ * array needs to start at zero.  The array's address is looked up on the first call on a device,
+ * for the device that is current in the calling thread: make that first call outside any graph
+ * capture, with the device of the pointers and of the stream current (as for every entry point
+ * here).                                                                                     */
 int64_t om_moe_sort_static_capacity_bytes(void);
 int om_moe_sort_static(const void *selected_experts, int index_dtype, int64_t T, int K,
                        int expert_start_idx, int expert_end_idx, int32_t *cum_token_counts,

@@ -198,6 +198,22 @@ static int adamw_launch(void *param, void *grad, float *master, float *exp_avg, 
     if (!om_aligned16(grad) || !om_aligned16(master) || !om_aligned16(exp_avg) ||
         !om_aligned16(exp_avg_sq) || (param_dtype == OM_BF16 && !om_aligned16(param)))
         return OM_ERR_ALIGN;
+    // One launch gives every lane one 4-element vector and the runtime takes fewer than 2^32 threads
+    // per launch, so buffers beyond 2^33 elements are updated in consecutive launches over
+    // sub-ranges (the update is element-wise: the same bits as one pass).
+    constexpr int64_t MAX_PER_LAUNCH = 1LL << 33;
+    if (n > MAX_PER_LAUNCH) {
+        const int64_t esz = param_dtype == OM_BF16 ? 2 : 4;
+        for (int64_t lo = 0; lo < n; lo += MAX_PER_LAUNCH) {
+            const int64_t len = n - lo < MAX_PER_LAUNCH ? n - lo : MAX_PER_LAUNCH;
+            const int rc = adamw_launch(param ? static_cast<char *>(param) + lo * esz : nullptr,
+                                        static_cast<char *>(grad) + lo * esz, master + lo, exp_avg + lo,
+                                        exp_avg_sq + lo, len, lr, beta1, beta2, eps, weight_decay, step,
+                                        param_dtype, grad_scale, clip, stream);
+            if (rc != OM_OK) return rc;
+        }
+        return OM_OK;
+    }
 
     // Scalars exactly as the reference forms them: Python doubles, narrowed to fp32 where they
     // meet an fp32 tensor (optimizers.py:193-202).
@@ -216,8 +232,7 @@ static int adamw_launch(void *param, void *grad, float *master, float *exp_avg, 
     hipStream_t st = om_stream(stream);
     const int64_t n_vec = n / 4;
     const int64_t blocks = (n_vec + ADAMW_THREADS - 1) / ADAMW_THREADS;
-    // one launch: the runtime takes fewer than 2^32 threads per launch (17e9 elements here)
-    if (blocks * ADAMW_THREADS >= (1LL << 32)) return OM_ERR_SHAPE;
+    if (blocks * ADAMW_THREADS >= (1LL << 32)) return OM_ERR_SHAPE;   // (not reached: see MAX_PER_LAUNCH)
     const dim3 grid(static_cast<unsigned>(blocks)), block(ADAMW_THREADS);
     if (param_dtype == OM_BF16) {
         uint16_t *p = static_cast<uint16_t *>(param), *g = static_cast<uint16_t *>(grad);

@@ -569,7 +569,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // wgrad: zero the A c-rows past the end of the expert's rows (after the loads have landed,
     // before the barrier).  B holds finite in-segment data there, so the products vanish.
     auto zero_tail = [&](int step, char *stage) {
-        if (EPI != EPI_WGRAD) return;
+        if (EPI != EPI_WGRAD || step >= loop_steps) return;   // (nothing was fetched for a step past the last)
         const int c0 = (step < steps_per_phase ? rotated(step) : step) * BK;
         if (c0 + BK <= c_len) return;
         char *sa = stage + wave * (A_LOADS * 1024);

@@ -445,13 +445,17 @@ __global__ __launch_bounds__(256) void balance_reduce_kernel(const float *__rest
                                                              float *__restrict__ count) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= N) return;
-    float ps = 0.0f, c = 0.0f;
+    float ps = 0.0f;
+    // a block's partial is a sum of at most BAL_TOKENS token weights (whole numbers for 0/1 weights
+    // and without weights); adding the partials in double keeps whole-number counts exact at any
+    // token count (a hot expert can exceed 2^24 tokens), one rounding to float at the end
+    double c = 0.0;
     for (int b = 0; b < n_blocks; b++) {
         ps += part_prob[static_cast<int64_t>(b) * N + i];
-        c += part_count[static_cast<int64_t>(b) * N + i];   // whole numbers below 2^24: exact
+        c += static_cast<double>(part_count[static_cast<int64_t>(b) * N + i]);
     }
     prob_sum[i] = ps;
-    count[i] = c;
+    count[i] = static_cast<float>(c);
 }
 
 // dlogits[t,i] = p_i * (g_i - sum_j p_j g_j): the softmax backward of sum_i g_i * p[t,i].

@@ -10,6 +10,8 @@ Pipeline of FastOlmoeParallelSparseMoeBlock.forward (reference moe.py:454-621):
 and the mirrored backward.  There is one code path: the reference's `use_triton_path_*` and
 `use_ref_path_*` switches are accepted where its signatures have them and ignored.
 """
+import warnings
+
 import torch
 import torch.nn as nn
 from torch.utils.checkpoint import checkpoint as torch_activation_checkpoint
@@ -17,6 +19,25 @@ from torch.utils.checkpoint import checkpoint as torch_activation_checkpoint
 import pcl_xpu_customops
 from optimus import _native as _n
 from optimus.profilers import record_pcl_function
+
+
+# Two of the blocks' fusions only take some operands (see gate_kernel_fits, routed_mlp_kernel_fits);
+# for the others the same block runs its unfused sequence of kernels from this library, whose bf16
+# roundings fall in other places.  That switch is announced once per reason (a UserWarning), or
+# refused when strict_fused_paths is set.
+strict_fused_paths = False
+_announced_switches = set()
+
+
+def note_unfused_path(what, why, instead="running the unfused sequence of kernels (same mathematics, bf16 "
+                                            "roundings in other places)"):
+    """Called where a block leaves a fused kernel path for the unfused sequence."""
+    message = f"{what}: {why}; {instead}"
+    if strict_fused_paths:
+        raise _n.NativeLibraryError(message + " [strict_fused_paths is set]")
+    if (what, why) not in _announced_switches:
+        _announced_switches.add((what, why))
+        warnings.warn(message, stacklevel=3)
 
 
 def get_tensor_list(tensor, cum_token_counts):
@@ -89,14 +110,25 @@ def _grouped_gemm(kind, a, b, out, cum, rows, G, N, K, w_stride, accumulate=Fals
 # ----------------------------------------------------------------------------------------------
 # Router
 # ----------------------------------------------------------------------------------------------
+def gate_kernel_unfit_reason(x, weight):
+    """None when the fused gate + routing kernel (om_router_gate_softmax_topk) takes these operands,
+    else why not."""
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
+        return f"operands are not bfloat16 device tensors ({x.dtype}, {weight.dtype})"
+    N, H = weight.shape
+    if N > 256:
+        return f"{N} experts (the kernel takes at most 256)"
+    if x.shape[0] == 0:
+        return "no tokens"
+    need = 512 if N <= 64 else 256 if N <= 128 else 64
+    if H % need != 0:
+        return f"hidden size {H} is not a multiple of {need} (needed with {N} experts)"
+    return None
+
+
 def gate_kernel_fits(x, weight):
     """Shapes and dtypes the fused gate + routing kernel takes (om_router_gate_softmax_topk)."""
-    if not (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
-        return False
-    N, H = weight.shape
-    if N > 256 or x.shape[0] == 0:
-        return False
-    return H % (512 if N <= 64 else 256 if N <= 128 else 64) == 0
+    return gate_kernel_unfit_reason(x, weight) is None
 
 
 def _require_gate_shape(weight, h_multiple, what):
@@ -200,7 +232,11 @@ def fp32_logits_with_passthrough(x, weight):
     is torch's own float32 linear and x comes back as it is."""
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         _n.require_cuda_contiguous(x.contiguous(), weight.contiguous())
-        _require_gate_shape(weight, 64, "gate projection")
+        # the weight gradient's kernel is the strictest of the three gate kernels: say so before
+        # the forward pass rather than in the middle of the backward pass
+        needs_wgrad = weight.requires_grad and torch.is_grad_enabled()
+        _require_gate_shape(weight, 128 if needs_wgrad else 64,
+                            "gate projection with a weight gradient" if needs_wgrad else "gate projection")
         return GateLogitsFunction.apply(x.contiguous(), weight.contiguous())
     if x.dtype == torch.float32 and weight.dtype == torch.float32:
         return torch.nn.functional.linear(x, weight), x
@@ -705,15 +741,25 @@ class GatheredGroupMLPFunction(torch.autograd.Function):
                 *_per_expert_grads(dwg, dwu, dwd, len(ctx.leaves[0])))
 
 
-def routed_mlp_kernel_fits(hidden_states, routing_weights, w_gate, w_down):
-    """True when RoutedMLPFunction's kernels take these operands: bf16 activations and expert
-    weights on the GPU, fp32 or bf16 routing weights, H and I multiples of 128."""
+def routed_mlp_unfit_reason(hidden_states, routing_weights, w_gate, w_down):
+    """None when RoutedMLPFunction's kernels take these operands (bf16 activations and expert
+    weights on the GPU, fp32 or bf16 routing weights, H and I multiples of 128), else why not."""
     G, I, H = w_gate.shape
-    return (hidden_states.is_cuda and hidden_states.dim() == 2
-            and hidden_states.dtype == torch.bfloat16 and w_gate.dtype == torch.bfloat16
-            and w_down.dtype == torch.bfloat16
-            and routing_weights.dtype in (torch.bfloat16, torch.float32)
-            and H % 128 == 0 and I % 128 == 0)
+    if not (hidden_states.is_cuda and hidden_states.dim() == 2):
+        return "the hidden states are not a 2-D device tensor"
+    if not (hidden_states.dtype == torch.bfloat16 and w_gate.dtype == torch.bfloat16
+            and w_down.dtype == torch.bfloat16):
+        return f"activations / expert weights are not bfloat16 ({hidden_states.dtype}, {w_gate.dtype})"
+    if routing_weights.dtype not in (torch.bfloat16, torch.float32):
+        return f"routing weights are {routing_weights.dtype}"
+    if H % 128 != 0 or I % 128 != 0:
+        return f"hidden size {H} / ffn size {I} are not multiples of 128"
+    return None
+
+
+def routed_mlp_kernel_fits(hidden_states, routing_weights, w_gate, w_down):
+    """True when RoutedMLPFunction's kernels take these operands."""
+    return routed_mlp_unfit_reason(hidden_states, routing_weights, w_gate, w_down) is None
 
 
 def _routed_mlp_forward(hidden_states, routing_weights, input_indices, cum_expert_counts_ep,
@@ -1172,7 +1218,10 @@ def expert_computation(hidden_states, routing_weights, selected_experts, expert_
 
 class FastOlmoeParallelSparseMoeBlock(nn.Module):
     """Reference moe.py:407-632.  forward(hidden_states [B,S,H]) ->
-    (final_hidden_states [B,S,H], router_logits [B*S,N] or None)."""
+    (final_hidden_states [B,S,H], router_logits [B*S,N] or None).
+
+    Limits of a bfloat16 block (a shape outside them raises, nothing falls back to a library):
+    at most 256 experts in the gate; hidden size a multiple of 128 and ffn size a multiple of 64."""
 
     def __init__(self, config, pmap=None):
         super().__init__()
@@ -1240,7 +1289,10 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
         if isinstance(self.experts, MergedMLP):
             weights = (self.experts.gate_proj_merged_weight, self.experts.up_proj_merged_weight,
                        self.experts.down_proj_merged_weight)
-            if not routed_mlp_kernel_fits(hidden_states, routing_weights, weights[0], weights[2]):
+            why = routed_mlp_unfit_reason(hidden_states, routing_weights, weights[0], weights[2])
+            if why is not None:
+                if hidden_states.dtype == torch.bfloat16:    # (float32 modules run unfused by design)
+                    note_unfused_path("routing weight inside the expert MLP", why)
                 return None
             return RoutedMLPFunction.apply(hidden_states, routing_weights, input_indices,
                                            cum_expert_counts_ep, output_indices, selected_experts_indices,
@@ -1248,7 +1300,10 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
                                            "merged_bound" if rows_is_bound else True, *weights)
         pack_expert_weights(self.experts)
         w0, d0 = self.experts[0].gate_proj.weight, self.experts[0].down_proj.weight
-        if not routed_mlp_kernel_fits(hidden_states, routing_weights, w0.unsqueeze(0), d0.unsqueeze(0)):
+        why = routed_mlp_unfit_reason(hidden_states, routing_weights, w0.unsqueeze(0), d0.unsqueeze(0))
+        if why is not None:
+            if hidden_states.dtype == torch.bfloat16:    # (float32 modules run unfused by design)
+                note_unfused_path("routing weight inside the expert MLP", why)
             return None
         mlp_params = []
         for expert in self.experts:
@@ -1266,7 +1321,11 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
     def forward(self, hidden_states, residual=None):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
         flat = hidden_states.reshape(-1, hidden_dim)
-        if self.router_logits_fp32 and gate_kernel_fits(flat, self.gate.weight):
+        gate_unfit = gate_kernel_unfit_reason(flat, self.gate.weight) if self.router_logits_fp32 else None
+        if self.router_logits_fp32 and gate_unfit is not None and flat.dtype == torch.bfloat16:
+            note_unfused_path("gate projection fused with the routing", gate_unfit,
+                              instead="running the projection and the routing as separate kernels (same fp32 logits)")
+        if self.router_logits_fp32 and gate_unfit is None:
             # the experts read the router function's pass-through of the hidden states, so that their
             # input gradient and the gate's are added in one kernel (GateSoftmaxTopkFunction)
             routing_weights, selected_experts, router_logits, flat = GateSoftmaxTopkFunction.apply(

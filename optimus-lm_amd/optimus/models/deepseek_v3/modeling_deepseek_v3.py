@@ -162,7 +162,11 @@ class DeepseekV3ParallelMoE(nn.Module):
                            output_indices, selected_experts_indices, cum_token_counts, residual,
                            rows_is_bound=False, with_shared=False):
         _moe.pack_expert_weights(self.experts)
-        if not self._routed_kernels_fit(hidden_states, routing_weights):
+        w0, d0 = self.experts[0].gate_proj.weight, self.experts[0].down_proj.weight
+        why = _moe.routed_mlp_unfit_reason(hidden_states, routing_weights, w0.unsqueeze(0), d0.unsqueeze(0))
+        if why is not None:
+            if hidden_states.dtype == torch.bfloat16:    # (float32 modules run unfused by design)
+                _moe.note_unfused_path("routing weight inside the expert MLP", why)
             return None
         params = []
         for expert in self.experts:

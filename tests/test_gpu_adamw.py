@@ -118,16 +118,21 @@ def test_optimizer_class_matches_kernel(cuda, oracle_lib):
     assert float(opt.flat_grad.abs().max()) == 0.0 and model[0].weight.grad.data_ptr() == opt.flat_grad.data_ptr()
 
 
-def test_full_size_int64_indexing(cuda, oracle_lib):
+@pytest.mark.parametrize("which", ["baseline_6.9e9", "beyond_one_launch"])
+def test_full_size_int64_indexing(cuda, oracle_lib, which):
     """BASELINE size (6.9e9 elements, 110 GB of state): a CPU-generated pattern of 2^22 elements is
     tiled over the flat buffers; every tile must then equal the oracle's result on the pattern.
-    Checked on tiles at the start, across the 2^31 and 2^32 element boundaries, and at the end."""
+    Checked on tiles at the start, across the 2^31 and 2^32 element boundaries, and at the end.
+    Second size: 2^33 + 2^22 + 5 elements (137 GB of state), more than one launch can take (a lane
+    owns 4 elements, a launch has fewer than 2^32 lanes): the library splits the buffer, checked
+    across the 2^33 boundary and on the 5-element tail."""
     import synthetic_configs as sc
     from optimus.optimizers import adamw_step_
-    n = sc.ADAMW["n"]
+    n = sc.ADAMW["n"] if which == "baseline_6.9e9" else (1 << 33) + (1 << 22) + 5
+    torch.cuda.empty_cache()
     free, _ = torch.cuda.mem_get_info()
-    if free < 120e9:
-        pytest.skip("needs 120 GB of free device memory")
+    if free < 16 * n * 1.06:
+        pytest.skip(f"needs {16 * n * 1.06 / 1e9:.0f} GB of free device memory")
     tile = 1 << 22
     st = _state(tile)
     reps = -(-n // tile)
@@ -141,7 +146,10 @@ def test_full_size_int64_indexing(cuda, oracle_lib):
     torch.cuda.synchronize()
     p, w, m, v = _run_oracle(st, 100, HP, oracle_lib)
     last_full = (n // tile - 1) * tile
-    for start in (0, (1 << 31) - tile, 1 << 31, (1 << 32) - tile, 1 << 32, last_full):
+    starts = [0, (1 << 31) - tile, 1 << 31, (1 << 32) - tile, 1 << 32, last_full]
+    if n > (1 << 33):
+        starts += [(1 << 33) - tile, 1 << 33]
+    for start in starts:
         sl = slice(start, start + tile)
         assert np.array_equal(dev["master"][sl].cpu().numpy().view(np.uint32), w.view(np.uint32)), start
         assert np.array_equal(dev["exp_avg_sq"][sl].cpu().numpy().view(np.uint32), v.view(np.uint32)), start
@@ -155,3 +163,5 @@ def test_full_size_int64_indexing(cuda, oracle_lib):
         e = min(n, s + (1 << 30))
         bad += int((dev["param"][s:e] != dev["master"][s:e].to(torch.bfloat16)).sum())
     assert bad == 0
+    del dev
+    torch.cuda.empty_cache()

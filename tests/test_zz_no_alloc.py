@@ -65,3 +65,46 @@ def test_static_sort_rejects_what_does_not_fit(cuda):
     # one table cell under the limit is taken
     T2 = 2048 * 1022 // K
     assert int(lib.om_moe_sort_workspace_bytes(T2, K, NR)) <= cap
+
+
+def test_static_sort_allocates_nothing_and_replays_from_a_graph(cuda):
+    """What the entry point is for: after one call outside any capture (which resolves the array's
+    address), further calls leave the device's free memory and torch's allocator untouched, and the
+    call can be recorded into a HIP graph; every replay on new inputs gives om_moe_sort's bits."""
+    from optimus import _native as n
+    lib = n.lib()
+    T, N, K, start, end = 4096, 64, 8, 16, 48
+    NR = end - start
+    se = routed_experts(T, N, K, seed=1).to(cuda).contiguous()
+    out = _outputs(T, K, NR, cuda)
+
+    def call():
+        n.check(lib.om_moe_sort_static(n.ptr(se), n.index_code(se), T, K, start, end,
+                                       *[n.ptr(t) for t in out], n.stream()), "om_moe_sort_static")
+    call()                                            # first call: outside capture
+    torch.cuda.synchronize()
+    free0, alloc0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for trial in range(3):
+        se.copy_(routed_experts(T, N, K, seed=10 + trial, skew=0.5 * trial).to(cuda))
+        for t in out:
+            t.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        want, _ = _both(se.clone(), start, end, cuda)      # eager work between the replays
+        for name, x, y in zip(("cum_token_counts", "cum_expert_counts_ep", "input_indices", "output_indices",
+                               "selected_experts_indices"), want, out):
+            assert torch.equal(x, y), (trial, name)
