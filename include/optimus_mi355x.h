@@ -177,7 +177,7 @@ int om_router_gate_logits_split(const void *x, const void *gate_weight, int64_t 
  * gradient of the logits.  x [T,H] bf16; dlogits [T,N] fp32, rounded to bf16 as it is loaded;
  * products accumulate in fp32 over token ranges and the partial sums are added in a fixed order
  * (deterministic).  dweight [N,H] in dweight_dtype (OM_BF16 / OM_F32).  N <= 256, H a multiple
- * of 128; other shapes return OM_ERR_SHAPE.
+ * of 8; other shapes return OM_ERR_SHAPE.
  * workspace: om_router_gate_wgrad_workspace_bytes(T,H,N) bytes of device memory, 16-byte
  * aligned (negative = error code).                                                        */
 int64_t om_router_gate_wgrad_workspace_bytes(int64_t T, int H, int N);
@@ -388,7 +388,10 @@ int om_rmsnorm_bwd(const void *dy, const void *h, const void *weight, const floa
  * w_stride: elements between the matrices of consecutive experts in `weight` /
  * `weight_grad`; 0 means densely packed (N*K, the merged [G,N,K] layout).  A larger stride
  * serves per-expert nn.Linear weights that sit at a constant pitch inside one flat buffer
- * (a multiple of 8 elements, else OM_ERR_ALIGN).  N and K must be multiples of 128.  Tensors
+ * (a multiple of 8 elements, else OM_ERR_ALIGN).  N and K must be multiples of 64 (the 256x256
+ * tile serves extents that are multiples of 256 with a contraction that is a multiple of 128, the
+ * 128x128 tile everything else, with a partial last tile where an extent is not a multiple of 128).
+ * Tensors
  * may exceed 2^31 elements (64-bit block-uniform bases, 32-bit offsets inside a tile); only a
  * source whose rows are fetched through an index (the *_gathered / *_weighted forms below) must
  * span fewer than 2^31 elements, e.g. 1M tokens of 2048.  fwd and dgrad (and the merged-MLP fusions below) keep

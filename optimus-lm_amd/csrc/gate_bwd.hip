@@ -88,7 +88,8 @@ __global__ __launch_bounds__(256) void gate_wgrad_kernel(const uint16_t *__restr
             const int q = j * 256 + tid;
             const int64_t t = t0 + q / (HT / 8);
             xq[j] = u32x4{0, 0, 0, 0};
-            if (t < t_end) xq[j] = *reinterpret_cast<const u32x4 *>(x + t * H + h0 + (q % (HT / 8)) * 8);
+            const int hc = h0 + (q % (HT / 8)) * 8;     // the last column slice may be partial
+            if (t < t_end && hc < H) xq[j] = *reinterpret_cast<const u32x4 *>(x + t * H + hc);
         }
 #pragma unroll
         for (int j = 0; j < DL; j++) {
@@ -142,13 +143,14 @@ __global__ __launch_bounds__(256) void gate_wgrad_kernel(const uint16_t *__restr
             }
         }
     }
-    float *out = partial + (static_cast<int64_t>(blockIdx.y) * n_real) * H + h0 + wave * 32 + (lane & 31);
+    const int h = h0 + wave * 32 + (lane & 31);
+    float *out = partial + (static_cast<int64_t>(blockIdx.y) * n_real) * H + h;
 #pragma unroll
     for (int b = 0; b < NB; b++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int n = b * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-            if (n < n_real) out[static_cast<int64_t>(n) * H] = acc[b][r];
+            if (n < n_real && h < H) out[static_cast<int64_t>(n) * H] = acc[b][r];
         }
 }
 
@@ -181,7 +183,8 @@ __global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float *__r
 // Token ranges: enough blocks to fill the chip twice over, at least two stages each.
 inline int gate_wgrad_splits(int64_t T, int H) {
     const int64_t stages = (T + TC - 1) / TC;
-    int64_t want = (2 * 256 + (H / HT) - 1) / (H / HT);   // ~2 blocks per CU
+    const int slices = (H + HT - 1) / HT;
+    int64_t want = (2 * 256 + slices - 1) / slices;   // ~2 blocks per CU
     if (want > stages / 2) want = stages / 2;
     if (want < 1) want = 1;
     if (want > 256) want = 256;
@@ -189,7 +192,7 @@ inline int gate_wgrad_splits(int64_t T, int H) {
 }
 
 inline bool gate_wgrad_shape_ok(int64_t T, int H, int N) {
-    return T >= 0 && H > 0 && H % HT == 0 && N >= 1 && N <= 256;
+    return T >= 0 && H > 0 && H % 8 == 0 && N >= 1 && N <= 256;   // 16-byte chunks of x
 }
 
 // ---- input gradient of the gate projection ---------------------------------------------------
@@ -350,7 +353,7 @@ extern "C" int om_router_gate_wgrad(const void *x, const float *dlogits, int64_t
     hipStream_t st = om_stream(stream);
     const int64_t stages = (T + TC - 1) / TC;
     const int64_t tokens_per_split = (stages + splits - 1) / splits * TC;
-    const dim3 grid(H / HT, splits);
+    const dim3 grid((H + HT - 1) / HT, splits);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
     float *ws = static_cast<float *>(workspace);
     if (N <= 32)

@@ -290,6 +290,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                       (GATHER == GATHER_WA && AKIND == STRIDED && EPI == EPI_WGRAD), "gather variants");
     static_assert(!ROWW || EPI == EPI_SWIGLU || EPI == EPI_SWIGLU_BWD, "row weights belong to the SwiGLU epilogues");
     constexpr int NW = WAVES_M * WAVES_N;
+    // The 128x128 tile takes output extents that are any multiple of 64: its last tile along an
+    // extent may be partial (loads past the extent are clamped, stores masked).  The 256x256 tile is
+    // only launched on whole tiles and carries none of that.
+    constexpr bool EDGE = BM == 128;
+    // Contraction steps are taken in pairs (static stage names).  The weight gradient, whose step
+    // count follows the expert's rows, and the 128x128 tile end an odd count with a single step; the
+    // 256x256 forward / input-gradient kernels are only launched on even counts.
+    constexpr bool ANY_STEPS = EPI == EPI_WGRAD || EDGE;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wavefront sub-tile
     constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 accumulators per wavefront
     constexpr int A_BYTES = TileBytes<AKIND, BM>::value;
@@ -399,7 +407,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         if (EPI == EPI_WGRAD) {
             // tiles are numbered expert-major: an XCD works on whole experts (all tiles of dW[g]
             // share the expert's rows of both operands)
-            const int tiles_n = p.n_cols / BN;
+            const int tiles_n = (p.n_cols + BN - 1) / BN;
             expert = logical / p.tiles_e;
             const int tile = logical - expert * p.tiles_e;
             const int tm = tile / tiles_n, tn = tile % tiles_n;
@@ -411,7 +419,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             c_len = p.cum[expert + 1] - c_begin;
         } else {
             constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
-            const int tiles_n = p.n_cols / BN_OUT;
+            const int tiles_n = (p.n_cols + BN_OUT - 1) / BN_OUT;
             const int tile_m = logical / tiles_n;
             const int tile_n = logical % tiles_n;
             rot_a = tile_n; rot_b = tile_m & 7;
@@ -429,9 +437,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         c_len = __builtin_amdgcn_readfirstlane(c_len);
         steps_per_phase = (c_len + BK - 1) / BK;
         total_steps = steps_per_phase * p.phases;
-        // the loop takes steps in pairs; fwd/dgrad counts are even (kc % 128 == 0), an odd weight-gradient
-        // count ends with a single step
-        loop_steps = (EPI == EPI_WGRAD) ? total_steps : ((total_steps + 1) & ~1);
+        loop_steps = ANY_STEPS ? total_steps : ((total_steps + 1) & ~1);
         rot = (rot_a + rot_b) % (steps_per_phase > 0 ? steps_per_phase : 1);
 #pragma unroll
         for (int i = 0; i < A_LOADS; i++) {
@@ -447,7 +453,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             } else {
                 constexpr int CPR = BM / 8;
                 const int ch = (lane_s % CPR) ^ ((a_crow[i] & 3) << 2);
-                a_off[i] = row_begin + ch * 8;  // + (contraction row within the step) * lda per step
+                // (a partial last tile: chunks past the extent re-read its last chunk; masked on store)
+                a_off[i] = EDGE ? min(row_begin + ch * 8, p.kc - 8) : row_begin + ch * 8;  // + (contraction row within the step) * lda per step
             }
         }
 #pragma unroll
@@ -456,20 +463,24 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             if (BKIND == CONTIG) {
                 const int row = grp * 8 + (lane_s >> 3);
                 const int ch = (lane_s & 7) ^ swz(row);
+                // output columns past n_cols (a partial last column tile) re-read the last one; their
+                // results are masked on store
+                const int n_last = EDGE ? p.n_cols - 1 - n0 : BN;
                 if (EPI == EPI_SWIGLU) {
                     // LDS rows alternate 32 gate rows / 32 up rows; the up matrix is B[1]
                     const int blk = row >> 5;
                     const int n = (blk >> 1) * 32 + (row & 31);
-                    b_off[i] = n * ldb32 + ch * 8;
+                    b_off[i] = min(n, n_last) * ldb32 + ch * 8;
                 } else {
-                    b_off[i] = row * ldb32 + ch * 8;
+                    b_off[i] = min(row, n_last) * ldb32 + ch * 8;
                 }
             } else {
                 constexpr int CPR = BN / 8;
                 const int ch = (lane_s % CPR) ^ ((b_crow[i] & 3) << 2);
+                const int col8 = EDGE ? min(ch * 8, p.n_cols - 8 - n0) : ch * 8;   // (partial last column tile, as above)
                 // fwd/dgrad: the lane's contraction row within a step never changes, so it is part of
                 // the offset; wgrad clamps the row into the expert's segment per step
-                b_off[i] = ch * 8 + (EPI == EPI_WGRAD ? 0 : b_crow[i] * ldb32);
+                b_off[i] = col8 + (EPI == EPI_WGRAD ? 0 : b_crow[i] * ldb32);
             }
         }
         // block-uniform parts of the addresses (scalar registers)
@@ -498,7 +509,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         const int ph = (step >= steps_per_phase) ? 1 : 0;  // at most two phases
         const int sp = step - ph * steps_per_phase;
         int c0 = (sp < steps_per_phase ? rotated(sp) : sp) * BK;
-        if (EPI != EPI_WGRAD && c0 > c_len - BK) c0 = c_len - BK;
+        if (!ANY_STEPS && c0 > c_len - BK) c0 = c_len - BK;
         // first contraction row that this step's STRIDED loads may touch, folded into the scalar base
         // (rows are clamped into the segment, so the base is clamped the same way)
         const int c_lo = (EPI == EPI_WGRAD) ? max(min(c0, c_len - 1), 0) : c0;
@@ -709,7 +720,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         if (wave == 0) build_tile_table<BM>(p.cum, p.n_experts, lane, tile_end, seg);
         __syncthreads();
         constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
-        total_tiles = __builtin_amdgcn_readfirstlane(tile_end[p.n_experts - 1]) * (p.n_cols / BN_OUT);
+        total_tiles = __builtin_amdgcn_readfirstlane(tile_end[p.n_experts - 1]) * ((p.n_cols + BN_OUT - 1) / BN_OUT);
     }
     const int nbx = gridDim.x / NUM_XCD;
     const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
@@ -743,8 +754,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         for (int j = 0; j < TN; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
-    // Steps are taken in pairs so the stage names are static; an odd step count (wgrad only: the
-    // host requires kc % 128 == 0 otherwise) ends with a single step.
+    // Steps are taken in pairs so the stage names are static; an odd step count ends with a single
+    // step.
     if (loop_steps > 0) {
         if (!prefetched) issue_loads(0, stage0);
         __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -755,7 +766,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         const int n_steps = loop_steps;
         for (int step = 0; step < n_steps; step += 2) {
             half_step(stage0, stage1, step);
-            if (EPI != EPI_WGRAD || step + 1 < n_steps) half_step(stage1, stage0, step + 1);
+            if (!ANY_STEPS || step + 1 < n_steps) half_step(stage1, stage0, step + 1);
         }
     }
     __syncthreads();  // the stages are dead: stage 1 becomes the strips, stage 0 the next tile's
@@ -812,6 +823,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     };
     const int col0 = (EPI == EPI_SWIGLU) ? e_n0 + (wn_e * WN) / 2 : e_n0 + wn_e * WN;   // first output column
     uint16_t *Cb = p.C + (EPI == EPI_WGRAD ? e_expert * p.strideC : 0);
+    // Rows this wavefront may touch in global memory: the expert's rows (the weight gradient: the
+    // rows of dW), none at all when its columns lie past the last output column (a partial last
+    // column tile; extents are multiples of 64, so whole wavefronts are in or out).
+    const int row_lim = !EDGE ? (EPI == EPI_WGRAD ? 0x7fffffff : e_row_end)
+                              : (col0 < p.n_cols) ? (EPI == EPI_WGRAD ? p.kc : e_row_end) : 0;
     // ROWW forward: the weights of this lane's row in every strip, fetched together up front
     float wrow_all[(ROWW && EPI == EPI_SWIGLU) ? TM : 1];
     if (ROWW && EPI == EPI_SWIGLU) {
@@ -834,7 +850,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             for (int it = 0; it < ITS; it++) {
                 const int q = it * 64 + lane_e;
                 const int64_t o = (m0 + q / CPRW) * p.ldc + col0 + (q % CPRW) * 8;
-                old_out[EPI == EPI_WGRAD ? it : 0] = *reinterpret_cast<const u32x4 *>(Cb + o);
+                if (m0 + q / CPRW < row_lim)
+                    old_out[EPI == EPI_WGRAD ? it : 0] = *reinterpret_cast<const u32x4 *>(Cb + o);
             }
         }
         if (EPI == EPI_SWIGLU) {
@@ -874,7 +891,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             for (int it = 0; it < ITS; it++) {
                 const int q = it * 64 + lane_e;
                 const int64_t m = m0 + q / CPRW;
-                if (m < e_row_end) {
+                if (m < row_lim) {
                     const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
                     // g and u have no reader after this one: keep them out of the caches (-1 to -3 %)
                     gq[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.G + o));
@@ -887,7 +904,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                 const int64_t m = m0 + q / CPRW;
                 float dot = 0.0f;   // ROWW: this lane's part of sum_i dh[m][i] * silu(g[m][i]) * u[m][i]
                 const float wr = ROWW ? __shfl(w_strip, q / CPRW, 64) : 1.0f;
-                if (m < e_row_end) {
+                if (m < row_lim) {
                     float dh[8], gv[8], uv[8], dg[8], du[8];
                     Elem<uint16_t>::unpack(strip_get(0, q / CPRW, q % CPRW), dh);
                     Elem<uint16_t>::unpack(gq[it], gv);
@@ -919,7 +936,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                     // the CPRW lanes of a row are neighbours: add them up in a fixed order and let
                     // the first one store the sum for this wavefront's column range
                     dot = lane_group_sum<CPRW>(dot);
-                    if (q % CPRW == 0 && m < e_row_end) p.row_dot[(col0 / COLS) * p.rows + m] = dot;
+                    if (q % CPRW == 0 && m < row_lim) p.row_dot[(col0 / COLS) * p.rows + m] = dot;
                 }
             }
         } else {
@@ -927,7 +944,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             for (int it = 0; it < ITS; it++) {
                 const int q = it * 64 + lane_e;
                 const int64_t m = m0 + q / CPRW;
-                if (EPI == EPI_WGRAD || m < e_row_end) {
+                if (m < row_lim) {
                     const int64_t o = m * p.ldc + col0 + (q % CPRW) * 8;
                     u32x4 v = strip_get(0, q / CPRW, q % CPRW);
                     if (EPI == EPI_WGRAD && acc_out) {
@@ -1001,7 +1018,7 @@ int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad f
     constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
     if (p.n_experts > MAX_EXPERTS) return OM_ERR_SHAPE;   // the tile table lives in LDS
     p.m_tiles_max = static_cast<int>((rows + BM - 1) / BM + p.n_experts);
-    const int64_t tiles = static_cast<int64_t>(p.m_tiles_max) * (p.n_cols / BN_OUT);
+    const int64_t tiles = static_cast<int64_t>(p.m_tiles_max) * ((p.n_cols + BN_OUT - 1) / BN_OUT);
     if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
     p.total_tiles = static_cast<int>(tiles);
     ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI, GATHER, ROWW>
@@ -1009,22 +1026,22 @@ int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad f
     return om_launch_status();
 }
 
-// The tile shape launch_rows_auto picks: 256x256 when the extents allow it, the experts hold enough
-// rows to fill such tiles, and there are enough of them for at least half the CUs (a tiny problem is
-// spread over more CUs by the 128x128 tile).
-template <int EPI> bool uses_big_tile(int n_cols, int n_experts, int64_t rows) {
+// The tile shape launch_rows_auto picks: 256x256 when the output columns are a whole number of such
+// tiles, the contraction a whole number of step pairs, the experts hold enough rows to fill them, and there are enough of them for at least half
+// the CUs (a tiny problem is spread over more CUs by the 128x128 tile).  The 128x128 tile takes any
+// extents that are multiples of 64: its last column tile may be partial.
+template <int EPI> bool uses_big_tile(int n_cols, int kc, int n_experts, int64_t rows) {
     constexpr int div = (EPI == EPI_SWIGLU) ? 2 : 1;
-    if (n_cols % (256 / div) != 0 || rows < static_cast<int64_t>(n_experts) * 192) return false;
+    if (n_cols % (256 / div) != 0 || kc % 128 != 0 || rows < static_cast<int64_t>(n_experts) * 192) return false;
     const int64_t tiles = ((rows + 255) / 256) * (n_cols / (256 / div));
-    return tiles * 2 >= device_cu_count() || n_cols % (128 / div) != 0;
+    return tiles * 2 >= device_cu_count();
 }
 
 template <int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = false>
 int launch_rows_auto(GemmParams &p, int64_t rows, hipStream_t st) {
-    constexpr int div = (EPI == EPI_SWIGLU) ? 2 : 1;
-    if (uses_big_tile<EPI>(p.n_cols, p.n_experts, rows))
+    if (uses_big_tile<EPI>(p.n_cols, p.kc, p.n_experts, rows))
         return launch_rows<256, 256, AKIND, BKIND, EPI, GATHER, ROWW>(p, rows, st);
-    if (p.n_cols % (128 / div) != 0) return OM_ERR_SHAPE;
+    if (p.n_cols % 64 != 0) return OM_ERR_SHAPE;
     return launch_rows<128, 128, AKIND, BKIND, EPI, GATHER, ROWW>(p, rows, st);
 }
 
@@ -1033,7 +1050,7 @@ int launch_rows_auto(GemmParams &p, int64_t rows, hipStream_t st) {
 extern "C" int om_grouped_gemm_fwd(const void *input, const void *weight, void *output,
                                    const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                    int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(N, 64) || !mult(K, 64)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!input || !weight || !output || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(input) || !om_aligned16(weight) || !om_aligned16(output)) return OM_ERR_ALIGN;
@@ -1053,7 +1070,7 @@ extern "C" int om_grouped_gemm_fwd(const void *input, const void *weight, void *
 extern "C" int om_grouped_gemm_dgrad(const void *output_grad, const void *weight, void *input_grad,
                                      const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                      int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(N, 64) || !mult(K, 64)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!output_grad || !weight || !input_grad || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(output_grad) || !om_aligned16(weight) || !om_aligned16(input_grad)) return OM_ERR_ALIGN;
@@ -1077,7 +1094,7 @@ namespace {
 int wgrad_launch(const void *output_grad, const void *input, const int32_t *index, int gather,
                  int64_t src_rows, void *weight_grad, const int32_t *cum_token_counts, int64_t rows, int G,
                  int N, int K, int64_t w_stride, void *stream, bool accumulate = false) {
-    if (rows < 0 || G < 1 || !mult(N, 128) || !mult(K, 128)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(N, 64) || !mult(K, 64)) return OM_ERR_SHAPE;
     // rows == 0 (nothing routed to these experts): the activations may be empty tensors without
     // storage; the launch then only writes zeros
     if (!weight_grad || !cum_token_counts || (rows > 0 && (!output_grad || !input))) return OM_ERR_NULL;
@@ -1100,7 +1117,7 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inde
     // 256x256 tiles unless they are too few to occupy half the CUs
     const bool big = N % 256 == 0 && K % 256 == 0 &&
                      static_cast<int64_t>(G) * (N / 256) * (K / 256) * 2 >= device_cu_count();
-    p.tiles_e = big ? (N / 256) * (K / 256) : (N / 128) * (K / 128);
+    p.tiles_e = big ? (N / 256) * (K / 256) : ((N + 127) / 128) * ((K + 127) / 128);
     const int64_t tiles = static_cast<int64_t>(p.tiles_e) * G;
     if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
     p.total_tiles = static_cast<int>(tiles);
@@ -1188,7 +1205,7 @@ int gate_up_fwd_launch(const void *x, const int32_t *x_rows, int64_t src_rows, c
                        const void *w_up, const float *row_weights, void *g, void *u, void *h,
                        const int32_t *cum_token_counts, int64_t rows, int G, int I, int H,
                        int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 128)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 64)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!x || !w_gate || !w_up || !g || !u || !h || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(x) || !om_aligned16(w_gate) || !om_aligned16(w_up) || !om_aligned16(g) ||
@@ -1258,7 +1275,7 @@ int down_dgrad_launch(const void *dy, const int32_t *dy_rows, int64_t src_rows, 
                       const void *g, const void *u, const float *row_weights, void *dg, void *du,
                       float *row_dot, const int32_t *cum_token_counts, int64_t rows, int G, int I, int H,
                       int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(I, 128) || !mult(H, 128)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 64)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!dy || !w_down || !g || !u || !dg || !du || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(dy) || !om_aligned16(w_down) || !om_aligned16(g) || !om_aligned16(u) ||
@@ -1315,7 +1332,7 @@ extern "C" int om_merged_mlp_gate_up_dgrad(const void *dg, const void *du, const
                                            const void *w_up, void *dx, const int32_t *cum_token_counts,
                                            int64_t rows, int G, int I, int H, int64_t w_stride,
                                            void *stream) {
-    if (rows < 0 || G < 1 || !mult(I, 128) || !mult(H, 128)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 64)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!dg || !du || !w_gate || !w_up || !dx || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(dg) || !om_aligned16(du) || !om_aligned16(w_gate) || !om_aligned16(w_up) ||

@@ -143,7 +143,7 @@ def _gate_weight_grad(x, weight, dlogits):
     """dweight[n,h] = sum_t dlogits[t,n] x[t,h]: a long contraction with a tiny output, split
     over token ranges on the device (om_router_gate_wgrad) instead of a library GEMM that would
     run on a few CUs."""
-    _require_gate_shape(weight, 128, "gate weight gradient")
+    _require_gate_shape(weight, 8, "gate weight gradient")
     T, (N, H) = x.shape[0], weight.shape
     lib = _n.lib()
     ws_bytes = lib.om_router_gate_wgrad_workspace_bytes(T, H, N)
@@ -232,11 +232,9 @@ def fp32_logits_with_passthrough(x, weight):
     is torch's own float32 linear and x comes back as it is."""
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         _n.require_cuda_contiguous(x.contiguous(), weight.contiguous())
-        # the weight gradient's kernel is the strictest of the three gate kernels: say so before
-        # the forward pass rather than in the middle of the backward pass
-        needs_wgrad = weight.requires_grad and torch.is_grad_enabled()
-        _require_gate_shape(weight, 128 if needs_wgrad else 64,
-                            "gate projection with a weight gradient" if needs_wgrad else "gate projection")
+        # the forward kernels are the strictest of the gate kernels (the two backward kernels take
+        # any hidden size that is a multiple of 8), so a shape that passes here passes in backward
+        _require_gate_shape(weight, 64, "gate projection")
         return GateLogitsFunction.apply(x.contiguous(), weight.contiguous())
     if x.dtype == torch.float32 and weight.dtype == torch.float32:
         return torch.nn.functional.linear(x, weight), x
@@ -743,7 +741,7 @@ class GatheredGroupMLPFunction(torch.autograd.Function):
 
 def routed_mlp_unfit_reason(hidden_states, routing_weights, w_gate, w_down):
     """None when RoutedMLPFunction's kernels take these operands (bf16 activations and expert
-    weights on the GPU, fp32 or bf16 routing weights, H and I multiples of 128), else why not."""
+    weights on the GPU, fp32 or bf16 routing weights, H and I multiples of 64), else why not."""
     G, I, H = w_gate.shape
     if not (hidden_states.is_cuda and hidden_states.dim() == 2):
         return "the hidden states are not a 2-D device tensor"
@@ -752,8 +750,8 @@ def routed_mlp_unfit_reason(hidden_states, routing_weights, w_gate, w_down):
         return f"activations / expert weights are not bfloat16 ({hidden_states.dtype}, {w_gate.dtype})"
     if routing_weights.dtype not in (torch.bfloat16, torch.float32):
         return f"routing weights are {routing_weights.dtype}"
-    if H % 128 != 0 or I % 128 != 0:
-        return f"hidden size {H} / ffn size {I} are not multiples of 128"
+    if H % 64 != 0 or I % 64 != 0:
+        return f"hidden size {H} / ffn size {I} are not multiples of 64"
     return None
 
 
@@ -1221,7 +1219,7 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
     (final_hidden_states [B,S,H], router_logits [B*S,N] or None).
 
     Limits of a bfloat16 block (a shape outside them raises, nothing falls back to a library):
-    at most 256 experts in the gate; hidden size a multiple of 128 and ffn size a multiple of 64."""
+    at most 256 experts in the gate; hidden size and ffn size multiples of 64."""
 
     def __init__(self, config, pmap=None):
         super().__init__()

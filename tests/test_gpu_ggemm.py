@@ -63,7 +63,11 @@ CASES = [# few rows per expert with extents that are multiples of 256 (skewed sm
          ("ragged", 150, 6000, 128, 128), ("empties", 200, 70000, 256, 256),
          # all the work in one expert: the weight gradient's work-balanced split of the tiles over the
          # XCDs then cuts that expert's tiles eight ways and the zero tiles of the others ride along
-         ("onehot", 70, 5000, 256, 512), ("onehot", 9, 3000, 512, 256), ("onehot", 2, 130, 128, 128)]
+         ("onehot", 70, 5000, 256, 512), ("onehot", 9, 3000, 512, 256), ("onehot", 2, 130, 128, 128),
+         # extents that are multiples of 64 but not of 128: partial last tiles along the output columns
+         # (and, for the weight gradient, along both extents of dW), odd numbers of contraction steps
+         ("ragged", 8, 1000, 320, 192), ("uniform", 4, 512, 64, 64), ("empties", 16, 777, 192, 448),
+         ("ragged", 64, 20000, 320, 2048), ("onehot", 5, 700, 2048, 320)]
 
 
 @pytest.mark.parametrize("kind,G,rows,N,K", CASES)
@@ -101,7 +105,10 @@ def test_grouped_gemm_fwd_dgrad_wgrad(cuda, kind, G, rows, N, K):
                                             # skewed small batches: a few rows per expert
                                             ("ragged", 64, 4096, 1024, 2048), ("empties", 32, 700, 256, 512),
                                             ("onehot", 8, 500, 128, 256), ("ragged", 40, 1000, 384, 256),
-                                            ("empties", 64, 4096, 1024, 2048), ("ragged", 2, 7, 128, 128)])
+                                            ("empties", 64, 4096, 1024, 2048), ("ragged", 2, 7, 128, 128),
+                                            # hidden / ffn sizes that are multiples of 64 only
+                                            ("ragged", 8, 1500, 192, 320), ("uniform", 4, 300, 64, 64),
+                                            ("empties", 16, 9000, 320, 1088)])
 def test_merged_mlp_fused(cuda, kind, G, rows, I, H):
     """MergedMLP (fused gate+up+SwiGLU, fused down-dgrad+SwiGLU-backward, dual dgrad) against the
     fp32 composition silu(x Wg^T) * (x Wu^T) Wd^T under autograd."""

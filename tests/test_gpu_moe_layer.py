@@ -99,6 +99,9 @@ def test_fast_block_fwd_bwd(cuda, name, scale):
     (257, 512, 128, 64, 8, True),      # about 32 rows per expert, a partial last 64-token stage
     (100, 512, 256, 130, 5, False),    # expert count that is no multiple of 32 or 64
     (640, 256, 384, 6, 3, True),       # ffn size a multiple of 128 but not of 256
+    (200, 320, 192, 8, 2, True),       # hidden and ffn sizes that are multiples of 64 only
+    (513, 192, 320, 16, 4, False),
+    (2048, 320, 704, 8, 2, False),     # the same with enough rows per expert for several row tiles
 ])
 def test_fast_block_odd_small_shapes(cuda, T, H, I, N, K, renorm):
     """Whole block, forward and backward, on sizes that exercise the edges of the tilings (single

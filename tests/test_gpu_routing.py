@@ -264,7 +264,10 @@ def test_gate_softmax_topk_backward(cuda):
                                        (777, 7168, 256, torch.float32), (64, 2048, 64, torch.float32),
                                        # expert counts that are no multiple of 32 or of 4
                                        (300, 256, 8, torch.bfloat16), (1000, 384, 60, torch.float32),
-                                       (500, 128, 130, torch.float32), (257, 512, 7, torch.float32)])
+                                       (500, 128, 130, torch.float32), (257, 512, 7, torch.float32),
+                                       # hidden sizes that end in a partial 128-column slice
+                                       (700, 192, 8, torch.bfloat16), (2048, 320, 64, torch.float32),
+                                       (333, 72, 5, torch.float32)])
 def test_gate_weight_grad_matches_fp32_matmul(cuda, T, H, N, wdt):
     """om_router_gate_wgrad against the product it replaces: dlogits rounded to bf16, multiplied in
     fp32.  The bf16 x bf16 products are exact in fp32, so only the order of the fp32 sum differs
@@ -366,10 +369,11 @@ def test_gate_shapes_without_a_kernel_raise(cuda):
     x = torch.zeros(16, 128, dtype=torch.bfloat16, device=cuda)
     with pytest.raises(NativeLibraryError):
         fp32_logits(x, torch.zeros(300, 128, dtype=torch.bfloat16, device=cuda))          # more than 256 experts
-    x = torch.zeros(16, 192, dtype=torch.bfloat16, device=cuda)
+    x = torch.zeros(16, 196, dtype=torch.bfloat16, device=cuda)
     with pytest.raises(NativeLibraryError):
-        _gate_backward(x, torch.zeros(8, 192, dtype=torch.bfloat16, device=cuda),
-                       torch.zeros(16, 8, device=cuda), (False, True))                      # weight gradient: H % 128
+        _gate_backward(x, torch.zeros(8, 196, dtype=torch.bfloat16, device=cuda),
+                       torch.zeros(16, 8, device=cuda), (False, True))                      # weight gradient: H % 8
+    x = torch.zeros(16, 192, dtype=torch.bfloat16, device=cuda)
     with pytest.raises(TypeError):
         fp32_logits(x, torch.zeros(8, 192, dtype=torch.float32, device=cuda))              # mixed dtypes
 

@@ -23,7 +23,8 @@ def _call(name, *args):
 # (kind, G, rows, N, K): both tile shapes (256x256 needs N, K multiples of 256 and enough tiles),
 # odd row counts (single trailing contraction step), experts without rows
 ABI_CASES = [("ragged", 64, 4096, 256, 512), ("empties", 16, 777, 128, 256), ("uniform", 8, 1000, 512, 256),
-             ("onehot", 9, 3000, 512, 256), ("ragged", 3, 5, 128, 128), ("ragged", 150, 6000, 128, 128)]
+             ("onehot", 9, 3000, 512, 256), ("ragged", 3, 5, 128, 128), ("ragged", 150, 6000, 128, 128),
+             ("ragged", 8, 1000, 192, 320)]   # partial last tiles along both extents of dW
 
 
 @pytest.mark.parametrize("kind,G,rows,N,K", ABI_CASES)
