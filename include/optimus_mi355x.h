@@ -185,6 +185,21 @@ int om_router_gate_wgrad(const void *x, const float *dlogits, int64_t T, int H, 
                          void *dweight, int dweight_dtype, void *workspace,
                          int64_t workspace_bytes, void *stream);
 
+/* The gate projection of a float32 module and its backward, replacing the nn.Linear behind
+ * `router_logits = self.gate(hidden_states)` (optimus/models/common/moe.py:456) where the block is
+ * kept in float32 (the reference's small CPU-runnable configuration): plain float32 products,
+ * sums in a fixed order (the weight gradient's sum over the tokens is kept in double and rounded
+ * once).  Any T, H, N <= 65535.  Parity path, not tuned.
+ *   om_router_gate_logits_f32 : logits[t,n]  = sum_h x[t,h] * gate_weight[n,h]
+ *   om_router_gate_dgrad_f32  : dx[t,h]      = sum_n dlogits[t,n] * gate_weight[n,h]
+ *   om_router_gate_wgrad_f32  : dweight[n,h] = sum_t dlogits[t,n] * x[t,h]                       */
+int om_router_gate_logits_f32(const float *x, const float *gate_weight, int64_t T, int H, int N,
+                              float *logits_out, void *stream);
+int om_router_gate_dgrad_f32(const float *dlogits, const float *gate_weight, int64_t T, int H, int N,
+                             float *dx, void *stream);
+int om_router_gate_wgrad_f32(const float *x, const float *dlogits, int64_t T, int H, int N,
+                             float *dweight, void *stream);
+
 /* om_router_gate_dgrad: gradient of the gate's input,
  *   dx[t,h] = (base[t,h] +) sum_n bf16(dlogits[t,n]) * gate_weight[n,h]
  * what autograd computes for the same nn.Linear (mm(dlogits, weight)), optionally with the

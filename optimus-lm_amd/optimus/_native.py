@@ -50,6 +50,9 @@ SIGNATURES = {
     "om_router_gate_wgrad": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p, c_int, c_void_p,
                                      c_i64, c_void_p]),
     "om_router_gate_dgrad": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p]),
+    "om_router_gate_logits_f32": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p, c_void_p]),
+    "om_router_gate_dgrad_f32": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p, c_void_p]),
+    "om_router_gate_wgrad_f32": (c_int, [c_void_p, c_void_p, c_i64, c_int, c_int, c_void_p, c_void_p]),
     "om_router_balance_workspace_bytes": (c_i64, [c_i64, c_int]),
     "om_router_balance_stats": (c_int, [c_void_p, c_int, c_i64, c_int, c_int, c_void_p, c_void_p,
                                         c_void_p, c_i64, c_void_p]),

@@ -225,11 +225,43 @@ class GateLogitsFunction(torch.autograd.Function):
         return _gate_backward(x, weight, dlogits, ctx.needs_input_grad, other_grad=x_grad)
 
 
+class GateLogitsF32Function(torch.autograd.Function):
+    """logits = x @ weight.T for a float32 gate (om_router_gate_logits_f32) with both backward
+    products (om_router_gate_dgrad_f32, om_router_gate_wgrad_f32): the float32 module's gate without
+    a library GEMM."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        _n.require_cuda_contiguous(x, weight)
+        T, (N, H) = x.shape[0], weight.shape
+        logits = torch.empty((T, N), dtype=torch.float32, device=x.device)
+        _n.check(_n.lib().om_router_gate_logits_f32(_n.ptr(x), _n.ptr(weight), T, H, N, _n.ptr(logits),
+                                                    _n.stream()), "om_router_gate_logits_f32")
+        ctx.save_for_backward(x, weight)
+        return logits
+
+    @staticmethod
+    def backward(ctx, dlogits):
+        x, weight = ctx.saved_tensors
+        T, (N, H) = x.shape[0], weight.shape
+        dlogits = dlogits.to(torch.float32).contiguous()
+        dx = dw = None
+        if ctx.needs_input_grad[0]:
+            dx = torch.empty_like(x)
+            _n.check(_n.lib().om_router_gate_dgrad_f32(_n.ptr(dlogits), _n.ptr(weight), T, H, N, _n.ptr(dx),
+                                                       _n.stream()), "om_router_gate_dgrad_f32")
+        if ctx.needs_input_grad[1]:
+            dw = torch.empty_like(weight)
+            _n.check(_n.lib().om_router_gate_wgrad_f32(_n.ptr(x), _n.ptr(dlogits), T, H, N, _n.ptr(dw),
+                                                       _n.stream()), "om_router_gate_wgrad_f32")
+        return dx, dw
+
+
 def fp32_logits_with_passthrough(x, weight):
     """(router logits in float32, x) from 2-D x [T,H] and weight [N,H] (the gate's nn.Linear weight).
     bf16 operands go through the gate kernels (at most 256 experts, H a multiple of 64; anything
     else raises), and the returned x is GateLogitsFunction's pass-through; a float32 module's gate
-    is torch's own float32 linear and x comes back as it is."""
+    runs on the plain float32 gate kernels (GateLogitsF32Function) and x comes back as it is."""
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         _n.require_cuda_contiguous(x.contiguous(), weight.contiguous())
         # the forward kernels are the strictest of the gate kernels (the two backward kernels take
@@ -237,7 +269,7 @@ def fp32_logits_with_passthrough(x, weight):
         _require_gate_shape(weight, 64, "gate projection")
         return GateLogitsFunction.apply(x.contiguous(), weight.contiguous())
     if x.dtype == torch.float32 and weight.dtype == torch.float32:
-        return torch.nn.functional.linear(x, weight), x
+        return GateLogitsF32Function.apply(x.contiguous(), weight.contiguous()), x
     raise TypeError(f"router gate: activations and weight must both be bfloat16 or both float32 "
                     f"(got {x.dtype}, {weight.dtype})")
 
@@ -251,9 +283,11 @@ def gate_logits(x, gate):
     """router_logits = gate(x) in the module's dtype (reference moe.py:456,
     modeling_olmoe.py:284) for 2-D x.  A bf16 gate runs on the gate kernels: the fp32-accumulated
     logits rounded once to bf16, which is what a bf16 linear layer returns (up to the order of the
-    fp32 sum).  A float32 module's gate is torch's own float32 linear."""
+    fp32 sum).  A float32 module's gate runs on the plain float32 gate kernels."""
     if x.dtype == torch.bfloat16 and gate.weight.dtype == torch.bfloat16:
         return fp32_logits(x, gate.weight).to(torch.bfloat16)
+    if x.dtype == torch.float32 and gate.weight.dtype == torch.float32 and x.is_cuda and gate.bias is None:
+        return fp32_logits(x, gate.weight)
     return gate(x)
 
 

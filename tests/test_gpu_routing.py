@@ -416,3 +416,27 @@ def test_masked_balance_loss_matches_the_reference_expression(cuda, L, B, S, N, 
     ones = load_balancing_loss_func(tuple(d.detach() for d in dev), N, K, attention_mask=torch.ones(B, S, device=cuda))
     plain = load_balancing_loss_func(tuple(d.detach() for d in dev), N, K)
     assert abs(float(ones) - float(plain)) <= 1e-6 * float(plain)
+
+
+@pytest.mark.parametrize("T,H,N", [(2048, 256, 8), (1, 7, 3), (777, 100, 130), (5000, 2048, 64)])
+def test_float32_gate_kernels_match_float64_products(cuda, T, H, N):
+    """The float32 module's gate (om_router_gate_logits_f32 and its two backward products) against
+    float64 products of the same float32 values: only the order of the float32 sums differs, so the
+    bound is a few float32 roundings of the absolute sum (the weight gradient, summed in double,
+    one rounding of the result)."""
+    from optimus.models.common.moe import GateLogitsF32Function
+    g = torch.Generator().manual_seed(T + H + N)
+    x = torch.randn(T, H, generator=g)
+    w = torch.randn(N, H, generator=g) * 0.1
+    dl = torch.randn(T, N, generator=g)
+    xd, wd = x.to(cuda).requires_grad_(True), w.to(cuda).requires_grad_(True)
+    logits = GateLogitsF32Function.apply(xd, wd)
+    logits.backward(dl.to(cuda))
+    eps = 2.0 ** -23
+    cases = (("logits", logits, x.double() @ w.double().t(), x.double().abs() @ w.double().abs().t(), 8.0),
+             ("dx", xd.grad, dl.double() @ w.double(), dl.double().abs() @ w.double().abs(), 8.0),
+             ("dw", wd.grad, dl.double().t() @ x.double(), dl.double().abs().t() @ x.double().abs(), 1.0))
+    for name, got, ref, absum, k in cases:
+        err = (got.detach().double().cpu() - ref).abs()
+        bound = k * eps * absum + 1e-30
+        assert bool((err <= bound).all()), (name, float((err / bound).max()))
