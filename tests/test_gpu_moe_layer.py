@@ -438,3 +438,25 @@ def test_dsv3_block_one_rank_share(cuda, ep_ind):
                            *LAYER_BARS["grad"], tag=f"{tag} dws{key[1:]}")
     # the router weight gets its gradient only through the K gathered scores of each token
     assert_bf16_parity(blk.gate.weight.grad, rwt.grad, *DSV3_GATE_BAR, tag=tag + " drouter_w")
+
+
+def test_unfused_paths_are_announced_or_refused(cuda):
+    """A shape the fused gate+routing kernel does not take makes the block run the projection and the
+    routing separately: announced once as a UserWarning, refused when strict_fused_paths is set."""
+    import warnings
+    from optimus._native import NativeLibraryError
+    from optimus.models.common import moe
+    inp = sc.moe_inputs("C1", scale_tokens=0.125)      # hidden 256 with 8 experts: not a multiple of 512
+    blk = _olmoe_block(inp, cuda)
+    x = inp["x"].to(cuda).view(1, inp["cfg"]["T"], inp["cfg"]["H"])
+    moe._announced_switches.clear()
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        blk(x); blk(x)
+    assert sum("gate projection fused with the routing" in str(w.message) for w in seen) == 1
+    moe.strict_fused_paths = True
+    try:
+        with pytest.raises(NativeLibraryError):
+            blk(x)
+    finally:
+        moe.strict_fused_paths = False

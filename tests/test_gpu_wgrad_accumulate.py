@@ -189,3 +189,23 @@ def test_fresh_gradients_without_a_live_buffer(cuda):
         _native.launch_log = None
     assert not any(nm.endswith("_accumulate") for nm in names)
     assert all(p.grad is not None for p in blk.parameters())
+
+
+def test_accumulation_under_activation_checkpointing(cuda):
+    """With the block's expert computation under torch's activation checkpoint (the reference's
+    use_activation_checkpointing bit 0, moe.py:430-432, :612-616) the recomputed forward's backward
+    still adds into the live gradient buffer, with the same bits as without checkpointing."""
+    from optimus.optimizers import MixedPrecisionAdamW
+    res = []
+    for ckpt in (False, True):
+        blk = _olmoe_block(cuda, True)
+        blk.use_activation_checkpointing_for_moe = ckpt
+        opt = MixedPrecisionAdamW(blk.parameters(), blk, lr=1e-3, dtype=torch.bfloat16, device=cuda)
+        g = torch.Generator().manual_seed(21)
+        opt.zero_grad()
+        for _ in range(2):
+            x = torch.randn(2, 128, 256, generator=g).to(torch.bfloat16).to(cuda).requires_grad_(True)
+            blk(x)[0].backward(torch.randn(2, 128, 256, generator=g).to(torch.bfloat16).to(cuda))
+        torch.cuda.synchronize()
+        res.append(opt.flat_grad.clone())
+    assert (bits(res[0]) == bits(res[1])).all() and float(res[0].float().abs().max()) > 0
