@@ -88,7 +88,6 @@ struct GemmParams {
     int m_tiles_max;            // fwd/dgrad: upper bound on row tiles
     int total_tiles;            // logical tiles of the launch (the blocks loop over them)
     int tiles_e;                // wgrad: tiles per expert
-    int accumulate;             // wgrad: C[g] = bf16(float(C[g]) + float(bf16(acc))) instead of C[g] = acc
 };
 
 typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_ptr;
@@ -283,8 +282,9 @@ __device__ __forceinline__ void wgrad_xcd_run(const int32_t *cum, int n_experts,
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE,
-          bool ROWW = false>
+          bool ROWW = false, bool ACCUM = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const GemmParams p) {
+    static_assert(!ACCUM || EPI == EPI_WGRAD, "only the weight gradient adds into its output");
     static_assert(GATHER == GATHER_NONE || (GATHER == GATHER_A && AKIND == CONTIG && EPI != EPI_WGRAD) ||
                       (GATHER == GATHER_B && BKIND == STRIDED && EPI == EPI_WGRAD) ||
                       (GATHER == GATHER_WA && AKIND == STRIDED && EPI == EPI_WGRAD), "gather variants");
@@ -838,22 +838,26 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         }
     }
     // Weight gradient added to what the output already holds (a gradient buffer that several
-    // backward passes accumulate into): the old values of a strip are fetched before the strip is
-    // turned around, and the sum is what an in-place bf16 `grad += dW` gives, two roundings.
-    const bool acc_out = EPI == EPI_WGRAD && p.accumulate != 0;
-    u32x4 old_out[EPI == EPI_WGRAD ? ITS : 1];
+    // backward passes accumulate into): the old values of a strip are fetched one strip ahead (two
+    // register sets), and the sum is what an in-place bf16 `grad += dW` gives, two roundings.
+    constexpr bool acc_out = ACCUM;
+    u32x4 old2[ACCUM ? 2 : 1][ACCUM ? ITS : 1];
+    auto load_old = [&](int i, int buf) {
+        const int64_t m0 = static_cast<int64_t>(e_row_begin) + wm_e * WM + i * 32;
+#pragma unroll
+        for (int it = 0; it < ITS; it++) {
+            const int q = it * 64 + lane_e;
+            const int64_t o = (m0 + q / CPRW) * p.ldc + col0 + (q % CPRW) * 8;
+            if (m0 + q / CPRW < row_lim)
+                old2[ACCUM ? buf : 0][ACCUM ? it : 0] = *reinterpret_cast<const u32x4 *>(Cb + o);
+        }
+    };
+    if (ACCUM) load_old(0, 0);
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int64_t m0 = static_cast<int64_t>(e_row_begin) + wm_e * WM + i * 32;  // first row of the strip
-        if (EPI == EPI_WGRAD && acc_out) {
-#pragma unroll
-            for (int it = 0; it < ITS; it++) {
-                const int q = it * 64 + lane_e;
-                const int64_t o = (m0 + q / CPRW) * p.ldc + col0 + (q % CPRW) * 8;
-                if (m0 + q / CPRW < row_lim)
-                    old_out[EPI == EPI_WGRAD ? it : 0] = *reinterpret_cast<const u32x4 *>(Cb + o);
-            }
-        }
+        if (ACCUM && i + 1 < TM) load_old(i + 1, (i + 1) & 1);
+        u32x4 *old_out = old2[ACCUM ? (i & 1) : 0];
         if (EPI == EPI_SWIGLU) {
             const float wrow = wrow_all[(ROWW && EPI == EPI_SWIGLU) ? i : 0];   // ROWW: h = w[row] * silu(g) * u, one rounding
 #pragma unroll
@@ -950,7 +954,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                     if (EPI == EPI_WGRAD && acc_out) {
                         float fresh[8], old[8];
                         Elem<uint16_t>::unpack(v, fresh);
-                        Elem<uint16_t>::unpack(old_out[EPI == EPI_WGRAD ? it : 0], old);
+                        Elem<uint16_t>::unpack(old_out[ACCUM ? it : 0], old);
 #pragma unroll
                         for (int x = 0; x < 4; x++)
                             v[x] = pack2_bf16(old[2 * x] + fresh[2 * x], old[2 * x + 1] + fresh[2 * x + 1]);
@@ -1112,7 +1116,6 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inde
         !fits_gather(src_rows * (gather == GATHER_WA ? N : K)))
         return OM_ERR_SHAPE;
     p.rows = rows; p.n_experts = G; p.n_cols = K; p.kc = N; p.phases = 1;
-    p.accumulate = accumulate ? 1 : 0;
     hipStream_t st = om_stream(stream);
     // 256x256 tiles unless they are too few to occupy half the CUs
     const bool big = N % 256 == 0 && K % 256 == 0 &&
@@ -1123,18 +1126,27 @@ int wgrad_launch(const void *output_grad, const void *input, const int32_t *inde
     p.total_tiles = static_cast<int>(tiles);
     const dim3 grid_big(persistent_blocks<256>(tiles)), block_big(Waves<256>::M * Waves<256>::N * 64);
     const dim3 grid_small(persistent_blocks<128>(tiles)), block_small(256);
-    if (big && gather == GATHER_NONE)
-        ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD><<<grid_big, block_big, 0, st>>>(p);
-    else if (big && gather == GATHER_B)
-        ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD, GATHER_B><<<grid_big, block_big, 0, st>>>(p);
-    else if (big)
-        ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD, GATHER_WA><<<grid_big, block_big, 0, st>>>(p);
-    else if (gather == GATHER_NONE)
-        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD><<<grid_small, block_small, 0, st>>>(p);
-    else if (gather == GATHER_B)
-        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD, GATHER_B><<<grid_small, block_small, 0, st>>>(p);
-    else
-        ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD, GATHER_WA><<<grid_small, block_small, 0, st>>>(p);
+    // ACCUM (C[g] = bf16(float(C[g]) + float(bf16(acc))) instead of C[g] = acc) is a template
+    // parameter: the plain kernels carry none of it
+#define OM_WGRAD(GATHER_KIND, ACC)                                                                               \
+    do {                                                                                                         \
+        if (big)                                                                                                 \
+            ggemm_kernel<256, 256, Waves<256>::M, Waves<256>::N, STRIDED, STRIDED, EPI_WGRAD, GATHER_KIND, false, \
+                         ACC><<<grid_big, block_big, 0, st>>>(p);                                                \
+        else                                                                                                     \
+            ggemm_kernel<128, 128, 2, 2, STRIDED, STRIDED, EPI_WGRAD, GATHER_KIND, false, ACC>                    \
+                <<<grid_small, block_small, 0, st>>>(p);                                                         \
+    } while (0)
+    if (accumulate) {
+        if (gather == GATHER_NONE) OM_WGRAD(GATHER_NONE, true);
+        else if (gather == GATHER_B) OM_WGRAD(GATHER_B, true);
+        else OM_WGRAD(GATHER_WA, true);
+    } else {
+        if (gather == GATHER_NONE) OM_WGRAD(GATHER_NONE, false);
+        else if (gather == GATHER_B) OM_WGRAD(GATHER_B, false);
+        else OM_WGRAD(GATHER_WA, false);
+    }
+#undef OM_WGRAD
     return om_launch_status();
 }
 }  // namespace
