@@ -284,11 +284,18 @@ def gate_logits(x, gate):
     modeling_olmoe.py:284) for 2-D x.  A bf16 gate runs on the gate kernels: the fp32-accumulated
     logits rounded once to bf16, which is what a bf16 linear layer returns (up to the order of the
     fp32 sum).  A float32 module's gate runs on the plain float32 gate kernels."""
+    return gate_logits_with_passthrough(x, gate)[0]
+
+
+def gate_logits_with_passthrough(x, gate):
+    """(gate_logits(x, gate), x), the second being the gate kernels' pass-through of x for a bf16
+    gate (see fp32_logits_with_passthrough) and x itself otherwise."""
     if x.dtype == torch.bfloat16 and gate.weight.dtype == torch.bfloat16:
-        return fp32_logits(x, gate.weight).to(torch.bfloat16)
+        logits, x = fp32_logits_with_passthrough(x, gate.weight)
+        return logits.to(torch.bfloat16), x
     if x.dtype == torch.float32 and gate.weight.dtype == torch.float32 and x.is_cuda and gate.bias is None:
-        return fp32_logits(x, gate.weight)
-    return gate(x)
+        return fp32_logits(x, gate.weight), x
+    return gate(x), x
 
 
 class GateSoftmaxTopkFunction(torch.autograd.Function):
@@ -1365,10 +1372,13 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
                 hidden_states.dtype)
             hidden_states = flat.view(batch_size, sequence_length, hidden_dim)
         else:
+            # (the experts are fed from the gate projection's pass-through here too: their input
+            # gradient is then added to the gate's inside om_router_gate_dgrad)
             if self.router_logits_fp32:
-                router_logits = fp32_logits(flat, self.gate.weight)
+                router_logits, flat = fp32_logits_with_passthrough(flat, self.gate.weight)
             else:
-                router_logits = gate_logits(flat, self.gate)
+                router_logits, flat = gate_logits_with_passthrough(flat, self.gate)
+            hidden_states = flat.view(batch_size, sequence_length, hidden_dim)
             routing_weights, selected_experts = SoftmaxTopkRouterFunction.apply(
                 router_logits.contiguous(), self.num_experts_per_tok, self.norm_topk_prob,
                 hidden_states.dtype)

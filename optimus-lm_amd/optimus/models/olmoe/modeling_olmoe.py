@@ -80,7 +80,8 @@ class OlmoeParallelSparseMoeBlock(nn.Module):
 
     def forward(self, hidden_states):
         batch_size, sequence_length, hidden_dim = hidden_states.shape
-        router_logits = _moe.gate_logits(hidden_states.reshape(-1, hidden_dim), self.gate)
+        router_logits, flat = _moe.gate_logits_with_passthrough(hidden_states.reshape(-1, hidden_dim), self.gate)
+        hidden_states = flat.view(batch_size, sequence_length, hidden_dim)    # see gate_logits_with_passthrough
         routing_weights, selected_experts = _moe.SoftmaxTopkRouterFunction.apply(
             router_logits.contiguous(), self.num_experts_per_tok, self.norm_topk_prob,
             hidden_states.dtype)
