@@ -162,7 +162,8 @@ int om_router_gate_logits(const void *x, const void *gate_weight, int64_t T, int
 
 /* om_router_gate_logits_split: the same projection as om_router_gate_logits for gates with many
  * experts (the DeepSeek-V3 router, 256 x 7168): 128 tokens and a slice of H per block, the weight
- * tile shared through LDS, the slices added in a fixed order.  N <= 256, H a multiple of 64.
+ * tile shared through LDS, the slices added in a fixed order.  N <= 256, H a multiple of 8 (a last
+ * step with fewer than 64 columns multiplies zero-filled token fragments).
  * workspace: om_router_gate_logits_split_workspace_bytes(T,H,N) bytes, 16-byte aligned
  * (negative = error code).  Same value as om_router_gate_logits up to the order of the sum.   */
 int64_t om_router_gate_logits_split_workspace_bytes(int64_t T, int H, int N);
@@ -403,9 +404,11 @@ int om_rmsnorm_bwd(const void *dy, const void *h, const void *weight, const floa
  * w_stride: elements between the matrices of consecutive experts in `weight` /
  * `weight_grad`; 0 means densely packed (N*K, the merged [G,N,K] layout).  A larger stride
  * serves per-expert nn.Linear weights that sit at a constant pitch inside one flat buffer
- * (a multiple of 8 elements, else OM_ERR_ALIGN).  N and K must be multiples of 64 (the 256x256
- * tile serves extents that are multiples of 256 with a contraction that is a multiple of 128, the
- * 128x128 tile everything else, with a partial last tile where an extent is not a multiple of 128).
+ * (a multiple of 8 elements, else OM_ERR_ALIGN).  N and K must be multiples of 8, the size of a
+ * 16-byte vector (the 256x256 tile serves extents that are multiples of 256 with a contraction that
+ * is a multiple of 128; the 128x128 tile everything else, with a partial last tile where an extent
+ * is not a multiple of 128 and a zero-filled last contraction step where the contraction length is
+ * not a multiple of 64).
  * Tensors
  * may exceed 2^31 elements (64-bit block-uniform bases, 32-bit offsets inside a tile); only a
  * source whose rows are fetched through an index (the *_gathered / *_weighted forms below) must
@@ -424,7 +427,7 @@ int om_grouped_gemm_wgrad(const void *output_grad, const void *input, void *weig
 
 /* The same three products for float32 modules (GroupedGemmFunction runs in the module's dtype,
  * moe.py:174-178, :201-210; the reference's small CPU-runnable configuration is float32): fp32
- * operands, fp32 MFMA accumulation, fp32 results.  N and K multiples of 64, w_stride a multiple
+ * operands, fp32 MFMA accumulation, fp32 results.  N and K multiples of 8, w_stride a multiple
  * of 4.  Built for parity at fp32 accuracy, not tuned.                                       */
 int om_grouped_gemm_fwd_f32(const float *input, const float *weight, float *output,
                             const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
@@ -500,7 +503,7 @@ int om_grouped_gemm_wgrad_gathered(const void *output_grad, const void *input,
  *                              [src_rows, N] read through output_grad_rows = input_indices [rows]
  *   om_merged_mlp_down_dgrad_weighted  : dh' = dfinal[dy_rows[r]] @ Wd[e];
  *                              row_dot[part][r] = sum over the part's 64 columns of dh' * silu(g) * u
- *                              (parts = om_merged_mlp_row_dot_parts(I) = I / 64, fp32 [parts, rows]);
+ *                              (parts = om_merged_mlp_row_dot_parts(I) = ceil(I / 64), fp32 [parts, rows]);
  *                              then as om_merged_mlp_down_dgrad with dh = row_weights[r] * dh'
  *   om_moe_row_weights_grad  : dw[t,k] = sum over parts (in order) of row_dot[part][pos]; entries of
  *                              pairs outside the expert window are not written (pre-zero them)   */

@@ -37,6 +37,9 @@ __global__ __launch_bounds__(256) void gate_logits_split_kernel(const uint16_t *
     const int64_t t0 = static_cast<int64_t>(blockIdx.x) * GT + wave * 32;
     const int h_begin = blockIdx.y * h_per_split;
     const int steps = h_per_split / GK;
+    // H is any multiple of 8: the last step of the last slice may hold fewer than 64 columns.  Its token
+    // fragments past the end are zeros, its weight loads past the end re-read the last 8 columns.
+    const int h_len = min(H - h_begin, h_per_split);
     // token fragment: lane l holds token t0 + l % 32, 8 consecutive h starting at 8 * (l / 32)
     int64_t ta = t0 + (lane & 31);
     if (ta >= T) ta = T - 1;                    // rows past the end: valid memory, result unused
@@ -52,10 +55,18 @@ __global__ __launch_bounds__(256) void gate_logits_split_kernel(const uint16_t *
         wp[i] = w + static_cast<int64_t>(src) * H + h_begin + ch * 8;
     }
     auto issue_w = [&](int s, int stage) {
+        const bool tail = (s + 1) * GK > h_len;          // block-uniform
+        const int chunks = (h_len - s * GK) >> 3;         // 8-column chunks the step holds
 #pragma unroll
-        for (int i = 0; i < W_LOADS; i++)
-            __builtin_amdgcn_global_load_lds((glb_ptr)(wp[i] + s * GK),
-                                             (lds_ptr)(ws[stage] + (wave * W_LOADS + i) * 1024), 16, 0, 0);
+        for (int i = 0; i < W_LOADS; i++) {
+            const uint16_t *src = wp[i] + s * GK;
+            if (tail) {
+                const int row = (wave * W_LOADS + i) * 8 + (lane >> 3);
+                const int ch = (lane & 7) ^ ((row >> 1) & 7);
+                src -= max(ch - (chunks - 1), 0) * 8;
+            }
+            __builtin_amdgcn_global_load_lds((glb_ptr)src, (lds_ptr)(ws[stage] + (wave * W_LOADS + i) * 1024), 16, 0, 0);
+        }
     };
     f32x16 acc[NB];
 #pragma unroll
@@ -64,6 +75,14 @@ __global__ __launch_bounds__(256) void gate_logits_split_kernel(const uint16_t *
         for (int r = 0; r < 16; r++) acc[b][r] = 0.0f;
     u32x4 xa[2][GK / 16];
     auto fetch_x = [&](int s, int buf) {
+        if ((s + 1) * GK > h_len) {                       // block-uniform
+#pragma unroll
+            for (int u = 0; u < GK / 16; u++) {
+                const bool inside = s * GK + u * 16 + (lane >> 5) * 8 < h_len;
+                xa[buf][u] = inside ? *reinterpret_cast<const u32x4 *>(xp + s * GK + u * 16) : u32x4{0, 0, 0, 0};
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < GK / 16; u++) xa[buf][u] = *reinterpret_cast<const u32x4 *>(xp + s * GK + u * 16);
     };
@@ -127,14 +146,15 @@ __global__ __launch_bounds__(256) void gate_logits_reduce_kernel(const float *__
 }
 
 inline bool gate_split_shape_ok(int64_t T, int H, int N) {
-    return T >= 0 && T <= 0x7fffffffLL && N >= 1 && N <= 256 && H >= GK && H % GK == 0;
+    return T >= 0 && T <= 0x7fffffffLL && N >= 1 && N <= 256 && H >= 8 && H % 8 == 0;
 }
 
 // Slices of H: enough blocks for one per CU when the token count alone does not give them, each
-// slice a whole number of 64-wide steps (the fp32 partials cost 8 B per logit and slice).
+// slice a whole number of 64-wide steps, the last of which may be partial (the fp32 partials cost
+// 8 B per logit and slice).
 inline int gate_split_count(int64_t T, int H) {
     const int64_t token_blocks = (T + GT - 1) / GT;
-    const int steps = H / GK;
+    const int steps = (H + GK - 1) / GK;
     int best = 1;
     for (int s = 1; s <= 16 && s <= steps; s++)
         if (steps % s == 0) {
@@ -165,7 +185,7 @@ extern "C" int om_router_gate_logits_split(const void *x, const void *gate_weigh
     const dim3 grid(static_cast<unsigned>((T + GT - 1) / GT), splits);
     const uint16_t *xp = static_cast<const uint16_t *>(x), *wp = static_cast<const uint16_t *>(gate_weight);
     float *ws = static_cast<float *>(workspace);
-    const int hps = H / splits;
+    const int hps = (H + GK - 1) / GK / splits * GK;   // a whole number of steps; the last slice may end early
     if (N <= 64) gate_logits_split_kernel<2><<<grid, dim3(256), 0, st>>>(xp, wp, T, H, N, hps, ws);
     else if (N <= 128) gate_logits_split_kernel<4><<<grid, dim3(256), 0, st>>>(xp, wp, T, H, N, hps, ws);
     else gate_logits_split_kernel<8><<<grid, dim3(256), 0, st>>>(xp, wp, T, H, N, hps, ws);

@@ -83,7 +83,7 @@ struct GemmParams {
     int64_t rows;               // allocated activation rows (upper bound of cum[G])
     int n_experts;
     int n_cols;                 // output columns (fwd/dgrad) — tiles along N = n_cols / BN_OUT
-    int kc;                     // contraction length per phase (fwd/dgrad), multiple of 64
+    int kc;                     // contraction length per phase (fwd/dgrad), multiple of 8
     int phases;                 // 1 or 2
     int m_tiles_max;            // fwd/dgrad: upper bound on row tiles
     int total_tiles;            // logical tiles of the launch (the blocks loop over them)
@@ -112,6 +112,10 @@ __device__ __forceinline__ int64_t uniform64(int64_t v) {
 // (counter SQ_LDS_BANK_CONFLICT = 0, 4 cycles per read); period 16, so rows 32 apart share it.
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 __device__ __forceinline__ int contig_off(int row, int ch) { return row * 128 + ((ch ^ swz(row)) << 4); }
+
+// The chunk (8 contraction indices) that lane `lane` of direct load `grp` of a CONTIG tile fetches: the
+// load fills LDS rows grp*8 .. grp*8+7, lane -> (row grp*8 + lane/8, position lane%8 = chunk ^ swz(row)).
+__device__ __forceinline__ int contig_chunk(int grp, int lane) { return (lane & 7) ^ ((grp * 4 + (lane >> 4)) & 7); }
 
 // ---- STRIDED tile: 64 c-rows x R rows-of-the-operand; R*2-byte c-rows; chunk position =
 //      chunk ^ ((crow & 3) << 2): the four c-rows a transposing read touches land in four
@@ -282,15 +286,18 @@ __device__ __forceinline__ void wgrad_xcd_run(const int32_t *cum, int n_experts,
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE,
-          bool ROWW = false, bool ACCUM = false>
+          bool ROWW = false, bool ACCUM = false, bool KTAIL = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const GemmParams p) {
     static_assert(!ACCUM || EPI == EPI_WGRAD, "only the weight gradient adds into its output");
+    // KTAIL: forward / input-gradient products whose contraction length is not a multiple of 64 (the last
+    // step of a phase is partial); a kernel of its own, so that the others carry none of its handling
+    static_assert(!KTAIL || (BM == 128 && EPI != EPI_WGRAD && AKIND == CONTIG), "partial last contraction step: 128x128 forward / input gradient");
     static_assert(GATHER == GATHER_NONE || (GATHER == GATHER_A && AKIND == CONTIG && EPI != EPI_WGRAD) ||
                       (GATHER == GATHER_B && BKIND == STRIDED && EPI == EPI_WGRAD) ||
                       (GATHER == GATHER_WA && AKIND == STRIDED && EPI == EPI_WGRAD), "gather variants");
     static_assert(!ROWW || EPI == EPI_SWIGLU || EPI == EPI_SWIGLU_BWD, "row weights belong to the SwiGLU epilogues");
     constexpr int NW = WAVES_M * WAVES_N;
-    // The 128x128 tile takes output extents that are any multiple of 64: its last tile along an
+    // The 128x128 tile takes output extents that are any multiple of 8: its last tile along an
     // extent may be partial (loads past the extent are clamped, stores masked).  The 256x256 tile is
     // only launched on whole tiles and carries none of that.
     constexpr bool EDGE = BM == 128;
@@ -510,6 +517,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         const int sp = step - ph * steps_per_phase;
         int c0 = (sp < steps_per_phase ? rotated(sp) : sp) * BK;
         if (!ANY_STEPS && c0 > c_len - BK) c0 = c_len - BK;
+        // KTAIL kernels take contraction lengths that are any multiple of 8: the last step of a phase
+        // may hold fewer than 64 indices.  Its loads past the end re-read the last valid 8 indices (c-row)
+        // instead, and the A slots they fill are zeroed in LDS before the step is multiplied (zero_tail).
+        const bool c_tail = KTAIL && c0 + BK > c_len;   // block-uniform
+        const int c_chunks = (c_len - c0) >> 3;                           // 8-index chunks the step holds
         // first contraction row that this step's STRIDED loads may touch, folded into the scalar base
         // (rows are clamped into the segment, so the base is clamped the same way)
         const int c_lo = (EPI == EPI_WGRAD) ? max(min(c0, c_len - 1), 0) : c0;
@@ -527,6 +539,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             uint32_t off;  // bytes from the step's scalar base
             if (AKIND == CONTIG) {
                 off = static_cast<uint32_t>(a_off[i] + c0) * 2u;
+                if (c_tail) off -= static_cast<uint32_t>(max(contig_chunk(wave_u * A_LOADS + i, lane) - (c_chunks - 1), 0)) * 16u;
             } else {
                 int c = c0 + a_crow[i];
                 if (EPI == EPI_WGRAD) c = min(c, c_len - 1);  // stay in the segment; zeroed below
@@ -544,6 +557,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
             uint32_t off;
             if (BKIND == CONTIG) {
                 off = static_cast<uint32_t>(b_off[i] + c0) * 2u;
+                if (c_tail) off -= static_cast<uint32_t>(max(contig_chunk(wave_u * B_LOADS + i, lane) - (c_chunks - 1), 0)) * 16u;
             } else {
                 if (GATHER == GATHER_B) {
                     off = static_cast<uint32_t>(b_off[i] + b_src[GATHER == GATHER_B ? i : 0] * ldb32) * 2u;
@@ -556,6 +570,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
                     int o = b_off[i];
                     asm volatile("" : "+v"(o));
                     off = static_cast<uint32_t>(o) * 2u;
+                    if (c_tail) off -= static_cast<uint32_t>(max(c0 + b_crow[i] - (c_len - 1), 0) * ldb32) * 2u;
                 }
             }
             // EPI_SWIGLU: a load covers 8 LDS rows inside one 32-row block, all gate or all up rows, so
@@ -580,7 +595,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // wgrad: zero the A c-rows past the end of the expert's rows (after the loads have landed,
     // before the barrier).  B holds finite in-segment data there, so the products vanish.
     auto zero_tail = [&](int step, char *stage) {
-        if (EPI != EPI_WGRAD || step >= loop_steps) return;   // (nothing was fetched for a step past the last)
+        if ((EPI != EPI_WGRAD && !KTAIL) || step >= loop_steps) return;   // (nothing was fetched for a step past the last)
+        if (EPI != EPI_WGRAD) {
+            // KTAIL: the last step of a phase holds fewer than 64 indices (A is CONTIG here): zero the
+            // chunks past the end
+            const int ph = (step >= steps_per_phase) ? 1 : 0;
+            const int c0 = rotated(step - ph * steps_per_phase) * BK;
+            if (c0 + BK <= c_len) return;
+            const int c_chunks = (c_len - c0) >> 3;
+            char *sa = stage + wave * (A_LOADS * 1024);
+#pragma unroll
+            for (int i = 0; i < A_LOADS; i++)
+                if (contig_chunk(wave_u * A_LOADS + i, lane) >= c_chunks)
+                    *reinterpret_cast<u32x4 *>(sa + i * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
+            return;
+        }
         const int c0 = (step < steps_per_phase ? rotated(step) : step) * BK;
         if (c0 + BK <= c_len) return;
         char *sa = stage + wave * (A_LOADS * 1024);
@@ -824,10 +853,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     const int col0 = (EPI == EPI_SWIGLU) ? e_n0 + (wn_e * WN) / 2 : e_n0 + wn_e * WN;   // first output column
     uint16_t *Cb = p.C + (EPI == EPI_WGRAD ? e_expert * p.strideC : 0);
     // Rows this wavefront may touch in global memory: the expert's rows (the weight gradient: the
-    // rows of dW), none at all when its columns lie past the last output column (a partial last
-    // column tile; extents are multiples of 64, so whole wavefronts are in or out).
+    // rows of dW), none at all for a lane whose 8 columns lie past the last output column (a partial
+    // last column tile; extents are multiples of 8, so a lane's 16-byte chunk is in or out as a whole).
     const int row_lim = !EDGE ? (EPI == EPI_WGRAD ? 0x7fffffff : e_row_end)
-                              : (col0 < p.n_cols) ? (EPI == EPI_WGRAD ? p.kc : e_row_end) : 0;
+                              : (col0 + (lane_e % (COLS / 8)) * 8 < p.n_cols) ? (EPI == EPI_WGRAD ? p.kc : e_row_end) : 0;
     // ROWW forward: the weights of this lane's row in every strip, fetched together up front
     float wrow_all[(ROWW && EPI == EPI_SWIGLU) ? TM : 1];
     if (ROWW && EPI == EPI_SWIGLU) {
@@ -1017,7 +1046,7 @@ template <int BM> struct Waves {
     static constexpr int N = (BM == 256) ? 4 : 2;    // 128x128: 2 x 2 wavefronts of 64x64
 };
 
-template <int BM, int BN, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = false>
+template <int BM, int BN, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = false, bool KTAIL = false>
 int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad family
     constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
     if (p.n_experts > MAX_EXPERTS) return OM_ERR_SHAPE;   // the tile table lives in LDS
@@ -1025,7 +1054,7 @@ int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad f
     const int64_t tiles = static_cast<int64_t>(p.m_tiles_max) * ((p.n_cols + BN_OUT - 1) / BN_OUT);
     if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
     p.total_tiles = static_cast<int>(tiles);
-    ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI, GATHER, ROWW>
+    ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI, GATHER, ROWW, false, KTAIL>
         <<<dim3(persistent_blocks<BM>(tiles)), dim3(Waves<BM>::M * Waves<BM>::N * 64), 0, st>>>(p);
     return om_launch_status();
 }
@@ -1033,7 +1062,8 @@ int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad f
 // The tile shape launch_rows_auto picks: 256x256 when the output columns are a whole number of such
 // tiles, the contraction a whole number of step pairs, the experts hold enough rows to fill them, and there are enough of them for at least half
 // the CUs (a tiny problem is spread over more CUs by the 128x128 tile).  The 128x128 tile takes any
-// extents that are multiples of 64: its last column tile may be partial.
+// extents and contraction lengths that are multiples of 8: its last column tile and its last
+// contraction step may be partial.
 template <int EPI> bool uses_big_tile(int n_cols, int kc, int n_experts, int64_t rows) {
     constexpr int div = (EPI == EPI_SWIGLU) ? 2 : 1;
     if (n_cols % (256 / div) != 0 || kc % 128 != 0 || rows < static_cast<int64_t>(n_experts) * 192) return false;
@@ -1045,7 +1075,8 @@ template <int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = f
 int launch_rows_auto(GemmParams &p, int64_t rows, hipStream_t st) {
     if (uses_big_tile<EPI>(p.n_cols, p.kc, p.n_experts, rows))
         return launch_rows<256, 256, AKIND, BKIND, EPI, GATHER, ROWW>(p, rows, st);
-    if (p.n_cols % 64 != 0) return OM_ERR_SHAPE;
+    if (p.n_cols % 8 != 0 || p.kc % 8 != 0) return OM_ERR_SHAPE;
+    if (p.kc % 64 != 0) return launch_rows<128, 128, AKIND, BKIND, EPI, GATHER, ROWW, true>(p, rows, st);
     return launch_rows<128, 128, AKIND, BKIND, EPI, GATHER, ROWW>(p, rows, st);
 }
 
@@ -1054,7 +1085,7 @@ int launch_rows_auto(GemmParams &p, int64_t rows, hipStream_t st) {
 extern "C" int om_grouped_gemm_fwd(const void *input, const void *weight, void *output,
                                    const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                    int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(N, 64) || !mult(K, 64)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(N, 8) || !mult(K, 8)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!input || !weight || !output || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(input) || !om_aligned16(weight) || !om_aligned16(output)) return OM_ERR_ALIGN;
@@ -1074,7 +1105,7 @@ extern "C" int om_grouped_gemm_fwd(const void *input, const void *weight, void *
 extern "C" int om_grouped_gemm_dgrad(const void *output_grad, const void *weight, void *input_grad,
                                      const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                      int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(N, 64) || !mult(K, 64)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(N, 8) || !mult(K, 8)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!output_grad || !weight || !input_grad || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(output_grad) || !om_aligned16(weight) || !om_aligned16(input_grad)) return OM_ERR_ALIGN;
@@ -1098,7 +1129,7 @@ namespace {
 int wgrad_launch(const void *output_grad, const void *input, const int32_t *index, int gather,
                  int64_t src_rows, void *weight_grad, const int32_t *cum_token_counts, int64_t rows, int G,
                  int N, int K, int64_t w_stride, void *stream, bool accumulate = false) {
-    if (rows < 0 || G < 1 || !mult(N, 64) || !mult(K, 64)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(N, 8) || !mult(K, 8)) return OM_ERR_SHAPE;
     // rows == 0 (nothing routed to these experts): the activations may be empty tensors without
     // storage; the launch then only writes zeros
     if (!weight_grad || !cum_token_counts || (rows > 0 && (!output_grad || !input))) return OM_ERR_NULL;
@@ -1217,7 +1248,7 @@ int gate_up_fwd_launch(const void *x, const int32_t *x_rows, int64_t src_rows, c
                        const void *w_up, const float *row_weights, void *g, void *u, void *h,
                        const int32_t *cum_token_counts, int64_t rows, int G, int I, int H,
                        int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 64)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(I, 8) || !mult(H, 8)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!x || !w_gate || !w_up || !g || !u || !h || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(x) || !om_aligned16(w_gate) || !om_aligned16(w_up) || !om_aligned16(g) ||
@@ -1287,7 +1318,7 @@ int down_dgrad_launch(const void *dy, const int32_t *dy_rows, int64_t src_rows, 
                       const void *g, const void *u, const float *row_weights, void *dg, void *du,
                       float *row_dot, const int32_t *cum_token_counts, int64_t rows, int G, int I, int H,
                       int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 64)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(I, 8) || !mult(H, 8)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!dy || !w_down || !g || !u || !dg || !du || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(dy) || !om_aligned16(w_down) || !om_aligned16(g) || !om_aligned16(u) ||
@@ -1324,8 +1355,8 @@ extern "C" int om_merged_mlp_down_dgrad(const void *dy, const void *w_down, cons
 }
 
 extern "C" int om_merged_mlp_row_dot_parts(int I) {
-    if (I < ROW_DOT_COLS || I % ROW_DOT_COLS != 0) return OM_ERR_SHAPE;
-    return I / ROW_DOT_COLS;
+    if (I < 8 || I % 8 != 0) return OM_ERR_SHAPE;
+    return (I + ROW_DOT_COLS - 1) / ROW_DOT_COLS;
 }
 
 extern "C" int om_merged_mlp_down_dgrad_weighted(const void *dy, const int32_t *dy_rows, int64_t src_rows,
@@ -1344,7 +1375,7 @@ extern "C" int om_merged_mlp_gate_up_dgrad(const void *dg, const void *du, const
                                            const void *w_up, void *dx, const int32_t *cum_token_counts,
                                            int64_t rows, int G, int I, int H, int64_t w_stride,
                                            void *stream) {
-    if (rows < 0 || G < 1 || !mult(I, 64) || !mult(H, 64)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult(I, 8) || !mult(H, 8)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!dg || !du || !w_gate || !w_up || !dx || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(dg) || !om_aligned16(du) || !om_aligned16(w_gate) || !om_aligned16(w_up) ||

@@ -30,31 +30,32 @@ struct F32Params {
     int accumulate;   // wgrad: C += product instead of C = product
 };
 
-// Fill tile[row][c] (64 x 16) from an operand.  CONTIG: element (row, c) at base[(r0+row)*ld + c0+c],
-// rows >= r_end read as zero.  STRIDED: element (row, c) at base[(c0+c)*ld + r0+row], c >= c_end
-// read as zero (r0+row is always inside the matrix: its extent is a multiple of 64).
+// Fill tile[row][c] (64 x 16) from an operand.  CONTIG: element (row, c) at base[(r0+row)*ld + c0+c];
+// STRIDED: element (row, c) at base[(c0+c)*ld + r0+row].  Rows >= r_end and contraction indices
+// >= c_end read as zero (extents are multiples of 4, so a float4 is inside or outside as a whole).
 template <int KIND>
 __device__ __forceinline__ void load_tile(float (*tile)[PITCH], const float *base, int64_t ld, int64_t r0,
                                           int64_t r_end, int64_t c0, int64_t c_end, int tid) {
     if (KIND == F_CONTIG) {
         const int row = tid >> 2, c4 = (tid & 3) * 4;
         f4 v = {0.f, 0.f, 0.f, 0.f};
-        if (r0 + row < r_end) v = *reinterpret_cast<const f4 *>(base + (r0 + row) * ld + c0 + c4);
+        if (r0 + row < r_end && c0 + c4 < c_end) v = *reinterpret_cast<const f4 *>(base + (r0 + row) * ld + c0 + c4);
         tile[row][c4] = v[0]; tile[row][c4 + 1] = v[1]; tile[row][c4 + 2] = v[2]; tile[row][c4 + 3] = v[3];
     } else {
         const int c = tid >> 4, row4 = (tid & 15) * 4;
         f4 v = {0.f, 0.f, 0.f, 0.f};
-        if (c0 + c < c_end) v = *reinterpret_cast<const f4 *>(base + (c0 + c) * ld + r0 + row4);
+        if (c0 + c < c_end && r0 + row4 < r_end) v = *reinterpret_cast<const f4 *>(base + (c0 + c) * ld + r0 + row4);
         tile[row4][c] = v[0]; tile[row4 + 1][c] = v[1]; tile[row4 + 2][c] = v[2]; tile[row4 + 3][c] = v[3];
     }
 }
 
-// One 64x64 tile: C[m0.., n0..] = sum over c in [c0, c1) of A(m, c) * B(n, c).
+// One 64x64 tile: C[m0.., n0..] = sum over c in [c0, c1) of A(m, c) * B(n, c); rows >= m_end and
+// columns >= n_end are not stored.
 template <int AKIND, int BKIND>
 __device__ __forceinline__ void tile_product(const float *A, int64_t lda, int64_t a_r0, int64_t a_rend,
                                              const float *B, int64_t ldb, int64_t b_r0, int64_t b_rend,
                                              int64_t c0, int64_t c1, float *C, int64_t ldc, int64_t m0,
-                                             int64_t m_end, int64_t n0, bool accumulate = false) {
+                                             int64_t m_end, int64_t n0, int64_t n_end, bool accumulate = false) {
     __shared__ float ta[TB][PITCH], tb[TB][PITCH];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
@@ -80,7 +81,9 @@ __device__ __forceinline__ void tile_product(const float *A, int64_t lda, int64_
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             f4 v = {acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
-            f4 *dst = reinterpret_cast<f4 *>(C + m * ldc + n0 + wn + q * 8 + (lane >> 5) * 4);
+            const int64_t n = n0 + wn + q * 8 + (lane >> 5) * 4;
+            if (n >= n_end) continue;
+            f4 *dst = reinterpret_cast<f4 *>(C + m * ldc + n);
             if (accumulate) v += *dst;
             *dst = v;
         }
@@ -106,10 +109,10 @@ __global__ __launch_bounds__(256) void ggemm_f32_rows_kernel(const F32Params p) 
     if (expert < 0) return;
     const int64_t m0 = s_begin, m_end = s_end, n0 = static_cast<int64_t>(blockIdx.y) * TB;
     const float *B = p.B + expert * p.strideB;
-    // fwd:   B = W[g] [n][k], operand rows n0.. (always inside), contraction k
+    // fwd:   B = W[g] [n][k], operand rows n0.., contraction k
     // dgrad: B = W[g] [c][col] with c the contraction index, operand rows n0..
-    tile_product<F_CONTIG, BKIND>(p.A, p.lda, m0, m_end, B, p.ldb, n0, n0 + TB, 0, p.kc, p.C, p.ldc, m0,
-                                  m_end, n0);
+    tile_product<F_CONTIG, BKIND>(p.A, p.lda, m0, m_end, B, p.ldb, n0, p.n_cols, 0, p.kc, p.C, p.ldc, m0,
+                                  m_end, n0, p.n_cols);
 }
 
 // blockIdx = (column tile of dW, row tile of dW, expert): dW[g][n][k] = sum_r dout[r][n] * in[r][k]
@@ -118,11 +121,13 @@ __global__ __launch_bounds__(256) void ggemm_f32_wgrad_kernel(const F32Params p)
     const int64_t r0 = p.cum[expert], r1 = p.cum[expert + 1];
     const int64_t n0 = static_cast<int64_t>(blockIdx.y) * TB, k0 = static_cast<int64_t>(blockIdx.x) * TB;
     float *C = p.C + expert * p.strideC;
-    tile_product<F_STRIDED, F_STRIDED>(p.A, p.lda, n0, n0 + TB, p.B, p.ldb, k0, k0 + TB, r0, r1, C, p.ldc,
-                                       n0, n0 + TB, k0, p.accumulate != 0);
+    const int64_t n_end = p.kc < n0 + TB ? p.kc : n0 + TB;   // rows of dW: the N extent
+    tile_product<F_STRIDED, F_STRIDED>(p.A, p.lda, n0, p.kc, p.B, p.ldb, k0, p.n_cols, r0, r1, C, p.ldc,
+                                       n0, n_end, k0, p.n_cols, p.accumulate != 0);
 }
 
-inline bool mult64(int64_t v) { return v > 0 && v % 64 == 0; }
+inline bool mult8(int64_t v) { return v > 0 && v % 8 == 0; }
+inline unsigned tiles_of(int v) { return static_cast<unsigned>((v + TB - 1) / TB); }
 inline bool fits31(int64_t v) { return v >= 0 && v < (1LL << 31); }
 
 }  // namespace
@@ -130,7 +135,7 @@ inline bool fits31(int64_t v) { return v >= 0 && v < (1LL << 31); }
 extern "C" int om_grouped_gemm_fwd_f32(const float *input, const float *weight, float *output,
                                        const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                        int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult64(N) || !mult64(K)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult8(N) || !mult8(K)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!input || !weight || !output || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(input) || !om_aligned16(weight) || !om_aligned16(output)) return OM_ERR_ALIGN;
@@ -142,15 +147,15 @@ extern "C" int om_grouped_gemm_fwd_f32(const float *input, const float *weight, 
     if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
     p.n_experts = G; p.n_cols = N; p.kc = K;
     const int64_t m_tiles = (rows + TB - 1) / TB + G;
-    if (m_tiles > 0x7fffffffLL || N / TB > 65535) return OM_ERR_SHAPE;
-    ggemm_f32_rows_kernel<F_CONTIG><<<dim3(static_cast<unsigned>(m_tiles), N / TB), dim3(256), 0, om_stream(stream)>>>(p);
+    if (m_tiles > 0x7fffffffLL || tiles_of(N) > 65535) return OM_ERR_SHAPE;
+    ggemm_f32_rows_kernel<F_CONTIG><<<dim3(static_cast<unsigned>(m_tiles), tiles_of(N)), dim3(256), 0, om_stream(stream)>>>(p);
     return om_launch_status();
 }
 
 extern "C" int om_grouped_gemm_dgrad_f32(const float *output_grad, const float *weight, float *input_grad,
                                          const int32_t *cum_token_counts, int64_t rows, int G, int N, int K,
                                          int64_t w_stride, void *stream) {
-    if (rows < 0 || G < 1 || !mult64(N) || !mult64(K)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || !mult8(N) || !mult8(K)) return OM_ERR_SHAPE;
     if (rows == 0) return OM_OK;
     if (!output_grad || !weight || !input_grad || !cum_token_counts) return OM_ERR_NULL;
     if (!om_aligned16(output_grad) || !om_aligned16(weight) || !om_aligned16(input_grad)) return OM_ERR_ALIGN;
@@ -162,8 +167,8 @@ extern "C" int om_grouped_gemm_dgrad_f32(const float *output_grad, const float *
     if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideB * G)) return OM_ERR_SHAPE;
     p.n_experts = G; p.n_cols = K; p.kc = N;
     const int64_t m_tiles = (rows + TB - 1) / TB + G;
-    if (m_tiles > 0x7fffffffLL || K / TB > 65535) return OM_ERR_SHAPE;
-    ggemm_f32_rows_kernel<F_STRIDED><<<dim3(static_cast<unsigned>(m_tiles), K / TB), dim3(256), 0, om_stream(stream)>>>(p);
+    if (m_tiles > 0x7fffffffLL || tiles_of(K) > 65535) return OM_ERR_SHAPE;
+    ggemm_f32_rows_kernel<F_STRIDED><<<dim3(static_cast<unsigned>(m_tiles), tiles_of(K)), dim3(256), 0, om_stream(stream)>>>(p);
     return om_launch_status();
 }
 
@@ -171,7 +176,7 @@ namespace {
 int wgrad_f32_launch(const float *output_grad, const float *input, float *weight_grad,
                      const int32_t *cum_token_counts, int64_t rows, int G, int N, int K, int64_t w_stride,
                      void *stream, bool accumulate) {
-    if (rows < 0 || G < 1 || G > 65535 || !mult64(N) || !mult64(K)) return OM_ERR_SHAPE;
+    if (rows < 0 || G < 1 || G > 65535 || !mult8(N) || !mult8(K)) return OM_ERR_SHAPE;
     if (!weight_grad || !cum_token_counts || (rows > 0 && (!output_grad || !input))) return OM_ERR_NULL;
     if (!om_aligned16(output_grad) || !om_aligned16(input) || !om_aligned16(weight_grad)) return OM_ERR_ALIGN;
     F32Params p = {};
@@ -179,10 +184,10 @@ int wgrad_f32_launch(const float *output_grad, const float *input, float *weight
     p.lda = N; p.ldb = K; p.ldc = K;
     p.strideC = w_stride ? w_stride : static_cast<int64_t>(N) * K;
     if (p.strideC % 4 != 0) return OM_ERR_ALIGN;
-    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideC * G) || N / TB > 65535) return OM_ERR_SHAPE;
+    if (!fits31(rows * K) || !fits31(rows * N) || !fits31(p.strideC * G) || tiles_of(N) > 65535) return OM_ERR_SHAPE;
     p.n_experts = G; p.n_cols = K; p.kc = N;
     p.accumulate = accumulate ? 1 : 0;
-    ggemm_f32_wgrad_kernel<<<dim3(K / TB, N / TB, G), dim3(256), 0, om_stream(stream)>>>(p);
+    ggemm_f32_wgrad_kernel<<<dim3(tiles_of(K), tiles_of(N), G), dim3(256), 0, om_stream(stream)>>>(p);
     return om_launch_status();
 }
 }  // namespace

@@ -259,14 +259,14 @@ class GateLogitsF32Function(torch.autograd.Function):
 
 def fp32_logits_with_passthrough(x, weight):
     """(router logits in float32, x) from 2-D x [T,H] and weight [N,H] (the gate's nn.Linear weight).
-    bf16 operands go through the gate kernels (at most 256 experts, H a multiple of 64; anything
+    bf16 operands go through the gate kernels (at most 256 experts, H a multiple of 8; anything
     else raises), and the returned x is GateLogitsFunction's pass-through; a float32 module's gate
     runs on the plain float32 gate kernels (GateLogitsF32Function) and x comes back as it is."""
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         _n.require_cuda_contiguous(x.contiguous(), weight.contiguous())
-        # the forward kernels are the strictest of the gate kernels (the two backward kernels take
-        # any hidden size that is a multiple of 8), so a shape that passes here passes in backward
-        _require_gate_shape(weight, 64, "gate projection")
+        # (the forward and the two backward kernels take the same shapes, so a shape that passes here
+        # passes in backward)
+        _require_gate_shape(weight, 8, "gate projection")
         return GateLogitsFunction.apply(x.contiguous(), weight.contiguous())
     if x.dtype == torch.float32 and weight.dtype == torch.float32:
         return GateLogitsF32Function.apply(x.contiguous(), weight.contiguous()), x
@@ -782,7 +782,7 @@ class GatheredGroupMLPFunction(torch.autograd.Function):
 
 def routed_mlp_unfit_reason(hidden_states, routing_weights, w_gate, w_down):
     """None when RoutedMLPFunction's kernels take these operands (bf16 activations and expert
-    weights on the GPU, fp32 or bf16 routing weights, H and I multiples of 64), else why not."""
+    weights on the GPU, fp32 or bf16 routing weights, H and I multiples of 8), else why not."""
     G, I, H = w_gate.shape
     if not (hidden_states.is_cuda and hidden_states.dim() == 2):
         return "the hidden states are not a 2-D device tensor"
@@ -791,8 +791,8 @@ def routed_mlp_unfit_reason(hidden_states, routing_weights, w_gate, w_down):
         return f"activations / expert weights are not bfloat16 ({hidden_states.dtype}, {w_gate.dtype})"
     if routing_weights.dtype not in (torch.bfloat16, torch.float32):
         return f"routing weights are {routing_weights.dtype}"
-    if H % 64 != 0 or I % 64 != 0:
-        return f"hidden size {H} / ffn size {I} are not multiples of 64"
+    if H % 8 != 0 or I % 8 != 0:
+        return f"hidden size {H} / ffn size {I} are not multiples of 8"
     return None
 
 
@@ -1260,7 +1260,7 @@ class FastOlmoeParallelSparseMoeBlock(nn.Module):
     (final_hidden_states [B,S,H], router_logits [B*S,N] or None).
 
     Limits of a bfloat16 block (a shape outside them raises, nothing falls back to a library):
-    at most 256 experts in the gate; hidden size and ffn size multiples of 64."""
+    at most 256 experts in the gate; hidden size and ffn size multiples of 8."""
 
     def __init__(self, config, pmap=None):
         super().__init__()

@@ -63,7 +63,7 @@ def test_routers(lib):
     assert lib.om_router_gate_logits(P, P, 8, 2048, 64, None, None) == NULL
     need = lib.om_router_gate_logits_split_workspace_bytes(8192, 7168, 256)
     assert need > 0 and need % 16 == 0
-    assert lib.om_router_gate_logits_split_workspace_bytes(8192, 7100, 256) == SHAPE     # H % 64
+    assert lib.om_router_gate_logits_split_workspace_bytes(8192, 7100, 256) == SHAPE     # H % 8
     assert lib.om_router_gate_logits_split_workspace_bytes(8192, 7168, 300) == SHAPE     # N > 256
     assert lib.om_router_gate_logits_split(P, P, 8192, 7168, 256, P, P, need - 1, None) == WORKSPACE
     assert lib.om_router_gate_logits_split(P, None, 8192, 7168, 256, P, P, need, None) == NULL
@@ -143,7 +143,8 @@ def test_combine_with_residual(lib):
 
 def test_grouped_gemms(lib):
     args = (131072, 64, 2048, 1024, 0, None)
-    assert lib.om_grouped_gemm_fwd(P, P, P, P, 131072, 64, 2000, 1024, 0, None) == SHAPE    # N % 64
+    assert lib.om_grouped_gemm_fwd(P, P, P, P, 131072, 64, 2004, 1024, 0, None) == SHAPE    # N % 8
+    assert lib.om_grouped_gemm_fwd(P, P, P, P, 131072, 64, 2048, 1020, 0, None) == SHAPE    # K % 8
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 0, 64, 2048, 1024, 0, None) == OK            # no rows
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 4096, 1025, 256, 256, 0, None) == SHAPE      # G > 1024 (LDS table)
     assert lib.om_grouped_gemm_fwd(P, None, P, P, *args) == NULL
@@ -152,12 +153,12 @@ def test_grouped_gemms(lib):
     assert lib.om_grouped_gemm_fwd(P, P, P, P, 4096, 64, 2048, 1024, 2048 * 1024 + 4, None) == ALIGN   # expert pitch % 8
     assert lib.om_grouped_gemm_dgrad(P, P, P, None, *args) == NULL
     assert lib.om_grouped_gemm_wgrad(P, P, P, P, 131072, 0, 2048, 1024, 0, None) == SHAPE   # G < 1
-    assert lib.om_merged_mlp_gate_up_fwd(P, P, P, P, P, P, P, 131072, 64, 1000, 2048, 0, None) == SHAPE
+    assert lib.om_merged_mlp_gate_up_fwd(P, P, P, P, P, P, P, 131072, 64, 1004, 2048, 0, None) == SHAPE
     assert lib.om_merged_mlp_gate_up_fwd(P, P, None, P, P, P, P, 131072, 64, 1024, 2048, 0, None) == NULL
     assert lib.om_merged_mlp_down_dgrad(P, P, P, P, P, ODD, P, 131072, 64, 1024, 2048, 0, None) == ALIGN
     assert lib.om_merged_mlp_gate_up_dgrad(P, P, P, P, None, P, 131072, 64, 1024, 2048, 0, None) == NULL
-    # float32 forms: N, K multiples of 64
-    assert lib.om_grouped_gemm_fwd_f32(P, P, P, P, 4096, 8, 96, 256, 0, None) == SHAPE
+    # float32 forms: N, K multiples of 8
+    assert lib.om_grouped_gemm_fwd_f32(P, P, P, P, 4096, 8, 100, 256, 0, None) == SHAPE
     assert lib.om_grouped_gemm_fwd_f32(P, P, P, P, 0, 8, 64, 256, 0, None) == OK
     assert lib.om_grouped_gemm_fwd_f32(P, P, P, None, 4096, 8, 64, 256, 0, None) == NULL
     assert lib.om_grouped_gemm_fwd_f32(P, P, P, P, 4096, 8, 64, 256, 64 * 256 + 2, None) == ALIGN   # pitch % 4
@@ -184,7 +185,7 @@ def test_routing_weight_folded_into_the_expert_mlp(lib):
     assert lib.om_merged_mlp_gate_up_fwd_weighted(P, P, 16384, P, P, None, P, P, P, P, *g) == NULL   # no weights
     assert lib.om_merged_mlp_gate_up_fwd_weighted(P, None, 16384, P, P, P, P, P, P, P, *g) == NULL   # no index
     assert lib.om_merged_mlp_gate_up_fwd_weighted(P, P, 0, P, P, P, P, P, P, P, *g) == SHAPE
-    assert lib.om_merged_mlp_gate_up_fwd_weighted(P, P, 16384, P, P, P, P, P, P, P, 131072, 64, 1000, 2048, 0, None) == SHAPE
+    assert lib.om_merged_mlp_gate_up_fwd_weighted(P, P, 16384, P, P, P, P, P, P, P, 131072, 64, 1004, 2048, 0, None) == SHAPE
     assert lib.om_merged_mlp_gate_up_fwd_weighted(P, None, 0, P, P, None, P, P, P, P, 0, 64, 1024, 2048, 0, None) == OK
     assert lib.om_sum_ggemm_output(P, None, P, None, P, 16384, 2048, BF16, None) == NULL
     assert lib.om_sum_ggemm_output(P, P, P, None, P, 16384, 2048, 7, None) == DTYPE
@@ -195,6 +196,7 @@ def test_routing_weight_folded_into_the_expert_mlp(lib):
     assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 1 << 21, P, P, P, *gw) == SHAPE   # indexed source of 2^31 elements or more
     assert lib.om_grouped_gemm_wgrad_gathered_out(P, P, 16384, P, ODD, P, *gw) == ALIGN
     assert lib.om_merged_mlp_row_dot_parts(1024) == 16
+    assert lib.om_merged_mlp_row_dot_parts(200) == 4      # partial last 64-column group
     assert lib.om_merged_mlp_row_dot_parts(100) == SHAPE
     assert lib.om_merged_mlp_down_dgrad_weighted(P, P, 16384, P, P, P, P, P, P, None, P, *g) == NULL   # no row_dot
     assert lib.om_merged_mlp_down_dgrad_weighted(P, P, 16384, P, P, P, None, P, P, P, P, *g) == NULL   # no weights

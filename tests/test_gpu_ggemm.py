@@ -67,7 +67,11 @@ CASES = [# few rows per expert with extents that are multiples of 256 (skewed sm
          # extents that are multiples of 64 but not of 128: partial last tiles along the output columns
          # (and, for the weight gradient, along both extents of dW), odd numbers of contraction steps
          ("ragged", 8, 1000, 320, 192), ("uniform", 4, 512, 64, 64), ("empties", 16, 777, 192, 448),
-         ("ragged", 64, 20000, 320, 2048), ("onehot", 5, 700, 2048, 320)]
+         ("ragged", 64, 20000, 320, 2048), ("onehot", 5, 700, 2048, 320),
+         # extents that are multiples of 8 only: partial 16-byte-chunk column masks in the last tile, a
+         # last contraction step with fewer than 64 indices (zero-filled in LDS), tiny extents
+         ("ragged", 8, 1000, 200, 136), ("uniform", 4, 512, 72, 40), ("empties", 16, 777, 8, 8),
+         ("ragged", 6, 900, 328, 1000), ("onehot", 5, 700, 1000, 328), ("ragged", 3, 50, 24, 264)]
 
 
 @pytest.mark.parametrize("kind,G,rows,N,K", CASES)
@@ -108,7 +112,10 @@ def test_grouped_gemm_fwd_dgrad_wgrad(cuda, kind, G, rows, N, K):
                                             ("empties", 64, 4096, 1024, 2048), ("ragged", 2, 7, 128, 128),
                                             # hidden / ffn sizes that are multiples of 64 only
                                             ("ragged", 8, 1500, 192, 320), ("uniform", 4, 300, 64, 64),
-                                            ("empties", 16, 9000, 320, 1088)])
+                                            ("empties", 16, 9000, 320, 1088),
+                                            # ... and of 8 only
+                                            ("ragged", 8, 1500, 200, 328), ("uniform", 4, 300, 8, 8),
+                                            ("empties", 16, 2000, 72, 1000), ("ragged", 5, 600, 1000, 72)])
 def test_merged_mlp_fused(cuda, kind, G, rows, I, H):
     """MergedMLP (fused gate+up+SwiGLU, fused down-dgrad+SwiGLU-backward, dual dgrad) against the
     fp32 composition silu(x Wg^T) * (x Wu^T) Wd^T under autograd."""
@@ -202,7 +209,10 @@ def test_gathered_merged_mlp_with_no_routed_rows(cuda):
 
 @pytest.mark.parametrize("kind,G,rows,N,K", [("uniform", 4, 512, 256, 128), ("ragged", 8, 1000, 192, 320),
                                             ("empties", 16, 777, 64, 64), ("ragged", 3, 5, 128, 64),
-                                            ("uniform", 8, 4096, 512, 256)])
+                                            ("uniform", 8, 4096, 512, 256),
+                                            # extents that are multiples of 8 only
+                                            ("ragged", 8, 1000, 200, 136), ("uniform", 4, 300, 8, 8),
+                                            ("empties", 6, 500, 72, 328)])
 def test_grouped_gemm_float32(cuda, kind, G, rows, N, K):
     """float32 modules (the reference's GroupedGemmFunction runs in the module's dtype): the fp32
     kernels against per-expert matmul in float64.  fp32 products and sums, so only the order of

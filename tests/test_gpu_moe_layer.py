@@ -102,6 +102,9 @@ def test_fast_block_fwd_bwd(cuda, name, scale):
     (200, 320, 192, 8, 2, True),       # hidden and ffn sizes that are multiples of 64 only
     (513, 192, 320, 16, 4, False),
     (2048, 320, 704, 8, 2, False),     # the same with enough rows per expert for several row tiles
+    (300, 328, 200, 8, 2, True),       # hidden and ffn sizes that are multiples of 8 only
+    (700, 72, 1000, 12, 3, False),
+    (64, 8, 8, 4, 2, True),            # the smallest sizes the kernels take
 ])
 def test_fast_block_odd_small_shapes(cuda, T, H, I, N, K, renorm):
     """Whole block, forward and backward, on sizes that exercise the edges of the tilings (single

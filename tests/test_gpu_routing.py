@@ -184,7 +184,9 @@ def _gate_inputs(T, H, N, seed):
                                    # more than 64 experts: the kernel that shares the weight tile
                                    # through LDS and splits H (odd step counts, padded expert rows,
                                    # a partial last 128-token block, one and several slices)
-                                   (8192, 7168, 256), (1000, 1024, 130), (129, 320, 96), (5, 64, 200)])
+                                   (8192, 7168, 256), (1000, 1024, 130), (129, 320, 96), (5, 64, 200),
+                                   # hidden sizes that are multiples of 8 only: a last step with fewer than 64 columns
+                                   (300, 72, 8), (129, 328, 96), (1000, 1000, 130), (5, 8, 200), (2048, 200, 64)])
 def test_gate_logits_match_fp32_matmul(cuda, T, H, N):
     """fp32 logits from bf16 operands: the products are exact, only the order of the fp32 sum differs
     from the CPU matmul of the up-cast operands."""
