@@ -290,7 +290,7 @@ def bench_other_configs(args, device, with_cpu, only=None):
     def gemm_ms(per):
         return sum(v for k, v in per.items() if k in GEMM_ENTRY_PRODUCTS)
 
-    def entry(T, ms, per, flops, weight_bytes=None, extra=None, bound="mfma"):
+    def entry(T, ms, per, flops, weight_bytes=None, extra=None, bound="mfma", traffic=None):
         g = gemm_ms(per)
         tflops = flops / (g * 1e-3) / 1e12
         e = {"ms_per_step": round(ms, 4), "tokens_per_s": round(T / (ms * 1e-3), 1),
@@ -305,7 +305,7 @@ def bench_other_configs(args, device, with_cpu, only=None):
             gbs = weight_bytes / (g * 1e-3) / 1e9
             e["roofline"] = {"bound": "hbm", "kernel": "all expert GEMM launches of the step (weight streaming)",
                              "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+                             "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": traffic}
         else:
             e["roofline"] = {"bound": "mfma", "kernel": "all expert GEMM launches of the step",
                              "achieved": round(tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
@@ -386,7 +386,8 @@ def bench_other_configs(args, device, with_cpu, only=None):
             "om_merged_mlp_gate_up_fwd_weighted": one_pass * 2 / 3, "om_grouped_gemm_fwd": one_pass / 3,
             "om_merged_mlp_down_dgrad_weighted": one_pass / 3, "om_merged_mlp_gate_up_dgrad": one_pass * 2 / 3,
             "om_grouped_gemm_wgrad_gathered": one_pass * 2 / 3, "om_grouped_gemm_wgrad_gathered_out": one_pass / 3}
-        out["C4"] = entry(c["T"], ms, per, flops, wbytes, bound="hbm", extra={
+        out["C4"] = entry(c["T"], ms, per, flops, wbytes, bound="hbm",
+                          traffic=measured_traffic_bytes("C4:all_expert_gemm_launches"), extra={
             "weight_stream_gb_per_s_by_entry_point": {
                 k: round(b / (per[k] * 1e-3) / 1e9, 1) for k, b in per_launch.items() if k in per},
             "graph_replay_ms_per_step": round(graph_ms, 4),
