@@ -247,8 +247,15 @@ def test_grouped_gemm_float32(cuda, kind, G, rows, N, K):
         assert float(wd.grad[empty.to(cuda)].abs().max()) == 0.0
 
 
+# sizes of the seeded sweeps: multiples of 128, and multiples of 8 only (partial last tiles along every
+# extent, a last contraction step with 8 to 56 indices)
+SWEEP_SIZES = {"multiples_of_128": ([128, 256, 384, 512, 1024], [128, 256, 384, 640, 1024]),
+               "multiples_of_8": ([8, 24, 72, 136, 200, 264, 328, 520, 1000], [8, 40, 72, 136, 200, 264, 328, 584, 1000])}
+
+
+@pytest.mark.parametrize("sizes", sorted(SWEEP_SIZES))
 @pytest.mark.parametrize("seed", list(range(24)))
-def test_grouped_gemm_random_shapes(cuda, seed):
+def test_grouped_gemm_random_shapes(cuda, seed, sizes):
     """Seeded sweep over expert counts, row counts and sizes: exercises the persistent-block
     partition (fewer tiles than blocks, remainders over the 8 XCDs, experts without rows, one or many
     tiles per expert) on both tile shapes, against per-expert fp32 matmul."""
@@ -256,8 +263,8 @@ def test_grouped_gemm_random_shapes(cuda, seed):
     rng = np.random.RandomState(1234 + seed)
     G = int(rng.choice([1, 2, 3, 7, 16, 33, 64, 70]))
     rows = int(rng.choice([1, 17, 255, 256, 257, 1000, 3333, 6000, 20000]))
-    N = int(rng.choice([128, 256, 384, 512, 1024]))
-    K = int(rng.choice([128, 256, 384, 640, 1024]))
+    N = int(rng.choice(SWEEP_SIZES[sizes][0]))
+    K = int(rng.choice(SWEEP_SIZES[sizes][1]))
     kind = ["uniform", "ragged", "empties"][seed % 3]
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(rows, K, generator=g).to(torch.bfloat16)
@@ -284,8 +291,9 @@ def test_grouped_gemm_random_shapes(cuda, seed):
         assert_bf16_parity(wd.grad, dw_ref, *ONE_ROUNDING, tag=f"ggemm_random{tag} wgrad")
 
 
+@pytest.mark.parametrize("sizes", sorted(SWEEP_SIZES))
 @pytest.mark.parametrize("seed", list(range(12)))
-def test_gathered_merged_mlp_random_shapes(cuda, seed):
+def test_gathered_merged_mlp_random_shapes(cuda, seed, sizes):
     """Seeded sweep of the bit-identity between the GEMMs that read tokens through input_indices and
     gather-then-GEMM, over token counts, top-k, expert windows and sizes."""
     from optimus.models.common.moe import (GatheredMergedMLPFunction, MergedMLPFunction,
@@ -295,8 +303,8 @@ def test_gathered_merged_mlp_random_shapes(cuda, seed):
     N = int(rng.choice([4, 8, 16, 64]))
     K = int(rng.choice([1, 2, min(4, N)]))
     T = int(rng.choice([5, 64, 300, 1024, 5000]))
-    H = int(rng.choice([128, 256, 384, 512]))
-    I = int(rng.choice([128, 256, 384]))
+    H = int(rng.choice([128, 256, 384, 512] if sizes == "multiples_of_128" else [8, 72, 200, 328, 520]))
+    I = int(rng.choice([128, 256, 384] if sizes == "multiples_of_128" else [8, 40, 136, 264]))
     start = int(rng.choice([0, N // 4]))
     end = int(rng.choice([N, max(start + 1, N - N // 4)]))
     G = end - start
