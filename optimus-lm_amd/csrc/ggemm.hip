@@ -286,12 +286,22 @@ __device__ __forceinline__ void wgrad_xcd_run(const int32_t *cum, int n_experts,
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE,
-          bool ROWW = false, bool ACCUM = false, bool KTAIL = false>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const GemmParams p) {
+          bool ROWW = false, bool ACCUM = false, bool KTAIL = false, bool REGLOAD = false>
+// (second launch bound: two wavefronts per SIMD, i.e. at most 256 registers, for the 128x128 tile, whose two
+// blocks per CU depend on it; the 256x256 tile's 8 wavefronts imply it already)
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BM == 128 ? 2 : 1) void ggemm_kernel(const GemmParams p) {
     static_assert(!ACCUM || EPI == EPI_WGRAD, "only the weight gradient adds into its output");
     // KTAIL: forward / input-gradient products whose contraction length is not a multiple of 64 (the last
     // step of a phase is partial); a kernel of its own, so that the others carry none of its handling
     static_assert(!KTAIL || (BM == 128 && EPI != EPI_WGRAD && AKIND == CONTIG), "partial last contraction step: 128x128 forward / input gradient");
+    // REGLOAD: forward / input-gradient products whose experts hold few rows, where a launch is a stream of
+    // weights that are used once.  Both operands go through registers instead of direct global->LDS loads: the
+    // weights (B) are fetched TWO contraction steps ahead into two register sets, the activations (A, which
+    // mostly hit in L2) one step ahead, and are written to the LDS stage that has become free before the
+    // barrier that ends a step.  With direct loads the look-ahead cannot exceed one step: the compiler
+    // waits for every outstanding load before a barrier, since it cannot tell which LDS bytes a direct load
+    // in flight will write.  Same LDS layout, same order of the sums: bit-identical results.
+    static_assert(!REGLOAD || (BM == 128 && EPI != EPI_WGRAD && !KTAIL), "register-staged operands: 128x128 forward / input gradient");
     static_assert(GATHER == GATHER_NONE || (GATHER == GATHER_A && AKIND == CONTIG && EPI != EPI_WGRAD) ||
                       (GATHER == GATHER_B && BKIND == STRIDED && EPI == EPI_WGRAD) ||
                       (GATHER == GATHER_WA && AKIND == STRIDED && EPI == EPI_WGRAD), "gather variants");
@@ -511,7 +521,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // Loads of contraction step `step` into `stage`.
     // Loads [lo, hi) of the step's list (A loads first, then B loads); lo and hi are constants
     // after unrolling.
+    u32x4 rb[REGLOAD ? 2 : 1][REGLOAD ? B_LOADS : 1];   // REGLOAD: B of steps s+1 and s+2 (set = step % 2)
+    u32x4 ra[REGLOAD ? A_LOADS : 1];                    //          A of step s+1
     auto issue_part = [&](int step, char *stage, int lo, int hi) {
+        if (REGLOAD) return;                               // (no direct loads in these kernels)
         if (step >= loop_steps) return;                    // nothing left to fetch for this tile
         const int ph = (step >= steps_per_phase) ? 1 : 0;  // at most two phases
         const int sp = step - ph * steps_per_phase;
@@ -582,6 +595,55 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     };
     constexpr int NL = A_LOADS + B_LOADS;
     auto issue_loads = [&](int step, char *stage) { issue_part(step, stage, 0, NL); };
+    // REGLOAD: the loads of a step into registers, and from there into an LDS stage.  The loads are issued
+    // unconditionally (past a tile's last step they re-read its last step, unused): inside a branch they
+    // would make the compiler wait for all loads at the join, and the look-ahead would be gone.
+    auto fetch_a = [&](int step) {
+        if (!REGLOAD) return;
+        step = min(step, loop_steps - 1);
+        const int ph = (step >= steps_per_phase) ? 1 : 0;
+        const int c0 = rotated(step - ph * steps_per_phase) * BK;
+        const char *Ap = reinterpret_cast<const char *>((p.phases > 1 && ph ? p.A[1] : p.A[0]) + uniform64(a_base));
+#pragma unroll
+        for (int i = 0; i < A_LOADS; i++)
+            ra[REGLOAD ? i : 0] = *reinterpret_cast<const u32x4 *>(Ap + static_cast<uint32_t>(a_off[i] + c0) * 2u);
+    };
+    auto fetch_b = [&](int step, int set) {
+        if (!REGLOAD) return;
+        step = min(step, loop_steps - 1);
+        const int ph = (step >= steps_per_phase) ? 1 : 0;
+        const int c0 = rotated(step - ph * steps_per_phase) * BK;
+        const int64_t b_step = uniform64(b_base + (BKIND == STRIDED ? static_cast<int64_t>(c_begin + c0) * p.ldb : 0));
+        const char *Bp = reinterpret_cast<const char *>(
+            ((EPI != EPI_SWIGLU && p.phases > 1 && ph) ? p.B[1] : p.B[0]) + b_step);
+        const char *Bup = reinterpret_cast<const char *>(p.B[1] + b_step);
+#pragma unroll
+        for (int i = 0; i < B_LOADS; i++) {
+            uint32_t off;
+            if (BKIND == CONTIG) {
+                off = static_cast<uint32_t>(b_off[i] + c0) * 2u;
+            } else {
+                int o = b_off[i];
+                asm volatile("" : "+v"(o));
+                off = static_cast<uint32_t>(o) * 2u;
+            }
+            const bool up_rows = EPI == EPI_SWIGLU && ((((wave_u * B_LOADS + i) * 8) >> 5) & 1);
+            rb[REGLOAD ? set : 0][REGLOAD ? i : 0] = *reinterpret_cast<const u32x4 *>((up_rows ? Bup : Bp) + off);
+        }
+    };
+    // (a wavefront writes the 1 KB blocks that its direct loads would fill: base + lane * 16)
+    auto commit_a = [&](int step, char *stage) {
+        if (!REGLOAD || step >= loop_steps) return;
+        char *sa = stage + wave * (A_LOADS * 1024) + lane * 16;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; i++) *reinterpret_cast<u32x4 *>(sa + i * 1024) = ra[REGLOAD ? i : 0];
+    };
+    auto commit_b = [&](int step, char *stage, int set) {
+        if (!REGLOAD || step >= loop_steps) return;
+        char *sb = stage + A_BYTES + wave * (B_LOADS * 1024) + lane * 16;
+#pragma unroll
+        for (int i = 0; i < B_LOADS; i++) *reinterpret_cast<u32x4 *>(sb + i * 1024) = rb[REGLOAD ? set : 0][REGLOAD ? i : 0];
+    };
     // The direct loads of a step are spread over the MFMAs of a whole step rather than issued in
     // one burst: the texture path of a CU accepts about one 1 KB load per wavefront every ~220
     // cycles, and a wavefront that has to wait for it cannot issue its MFMAs meanwhile.  Shares of
@@ -717,25 +779,33 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
         __builtin_amdgcn_sched_barrier(0);
     };
     auto interleave = [&]() { interleave_loads(0); };
-    // one contraction step on `cur`; `nxt` holds step s+1 when this returns
-    auto half_step = [&](char *cur, char *nxt, int s) {
+    // one contraction step on `cur`; `nxt` holds step s+1 when this returns (par = s % 2)
+    auto half_step = [&](char *cur, char *nxt, int s, int par) {
 #pragma unroll
         for (int kk = 0; kk < BK / 16 - 1; kk++) {
             // the rest of the loads of step s+1 (their stage was released in the previous step)
             const int lo = LD_T + (kk > 0 ? LD_0 : 0) + (kk > 1 ? LD_1 : 0);
             const int n = kk == 0 ? LD_0 : (kk == 1 ? LD_1 : LD_2);
             issue_part(s + 1, nxt, lo, lo + n);
+            // REGLOAD: B of step s+2 into the register set that held B of step s (written to LDS a step ago);
+            // issued after the A loads of step s+1 (below, behind the barrier of the previous step), so that
+            // the wait for those leaves these in flight
+            if (REGLOAD && kk == 0) fetch_b(s + 2, par);
             read_group(cur, kk + 1, (kk + 1) & 1);
             mfma_group(kk & 1);
-            if (n > 0) interleave_loads(n); else interleave();
+            if (REGLOAD) { if (kk == 0) interleave_loads(B_LOADS); else interleave(); }
+            else if (n > 0) interleave_loads(n); else interleave();
         }
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's loads of step s+1 landed
+        if (!REGLOAD) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's loads of step s+1 landed
+        commit_a(s + 1, nxt);                // (REGLOAD: the compiler's own waits: all loads but the B_LOADS youngest)
+        commit_b(s + 1, nxt, par ^ 1);
         zero_tail(s + 1, nxt);
         __syncthreads();                     // everyone's did, and nobody reads `cur` any more
         issue_part(s + 2, cur, 0, LD_T);
+        fetch_a(s + 2);
         read_group(nxt, 0, 0);
         mfma_group((BK / 16 - 1) & 1);
-        if (LD_T > 0) interleave_loads(LD_T); else interleave();
+        if (REGLOAD) interleave_loads(A_LOADS); else if (LD_T > 0) interleave_loads(LD_T); else interleave();
     };
     // ---- persistent block: walks its share of the logical tiles --------------------------------
     // Hardware places block b on XCD b % 8.  XCD x owns the contiguous run [x*per, (x+1)*per) of
@@ -786,16 +856,19 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     // Steps are taken in pairs so the stage names are static; an odd step count ends with a single
     // step.
     if (loop_steps > 0) {
-        if (!prefetched) issue_loads(0, stage0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+        if (!prefetched) { issue_loads(0, stage0); fetch_a(0); fetch_b(0, 0); fetch_b(1, 1); }
+        if (!REGLOAD) __builtin_amdgcn_s_waitcnt(0x0F70);
+        commit_a(0, stage0);
+        commit_b(0, stage0, 0);
         zero_tail(0, stage0);
         __syncthreads();
         issue_part(1, stage1, 0, LD_T);
+        fetch_a(1);
         read_group(stage0, 0, 0);
         const int n_steps = loop_steps;
         for (int step = 0; step < n_steps; step += 2) {
-            half_step(stage0, stage1, step);
-            if (!ANY_STEPS || step + 1 < n_steps) half_step(stage1, stage0, step + 1);
+            half_step(stage0, stage1, step, 0);
+            if (!ANY_STEPS || step + 1 < n_steps) half_step(stage1, stage0, step + 1, 1);
         }
     }
     __syncthreads();  // the stages are dead: stage 1 becomes the strips, stage 0 the next tile's
@@ -806,7 +879,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void ggemm_kernel(const Gemm
     const int e_expert = expert, e_row_begin = row_begin, e_row_end = row_end, e_n0 = n0;
     have = next_tile();
     prefetched = have && loop_steps > 0;
-    if (prefetched) issue_loads(0, stage0);
+    if (prefetched) { issue_loads(0, stage0); fetch_a(0); fetch_b(0, 0); fetch_b(1, 1); }
 
     // ---- epilogue ------------------------------------------------------------------------------
     // Accumulator element r of lane l is output row (l % 32), column (r/4)*8 + (l/32)*4 + (r%4) of
@@ -1046,7 +1119,8 @@ template <int BM> struct Waves {
     static constexpr int N = (BM == 256) ? 4 : 2;    // 128x128: 2 x 2 wavefronts of 64x64
 };
 
-template <int BM, int BN, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = false, bool KTAIL = false>
+template <int BM, int BN, int AKIND, int BKIND, int EPI, int GATHER = GATHER_NONE, bool ROWW = false, bool KTAIL = false,
+          bool REGLOAD = false>
 int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad family
     constexpr int BN_OUT = (EPI == EPI_SWIGLU) ? BN / 2 : BN;
     if (p.n_experts > MAX_EXPERTS) return OM_ERR_SHAPE;   // the tile table lives in LDS
@@ -1054,7 +1128,7 @@ int launch_rows(GemmParams &p, int64_t rows, hipStream_t st) {  // fwd / dgrad f
     const int64_t tiles = static_cast<int64_t>(p.m_tiles_max) * ((p.n_cols + BN_OUT - 1) / BN_OUT);
     if (tiles > 0x7fffffffLL) return OM_ERR_SHAPE;
     p.total_tiles = static_cast<int>(tiles);
-    ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI, GATHER, ROWW, false, KTAIL>
+    ggemm_kernel<BM, BN, Waves<BM>::M, Waves<BM>::N, AKIND, BKIND, EPI, GATHER, ROWW, false, KTAIL, REGLOAD>
         <<<dim3(persistent_blocks<BM>(tiles)), dim3(Waves<BM>::M * Waves<BM>::N * 64), 0, st>>>(p);
     return om_launch_status();
 }
@@ -1077,6 +1151,11 @@ int launch_rows_auto(GemmParams &p, int64_t rows, hipStream_t st) {
         return launch_rows<256, 256, AKIND, BKIND, EPI, GATHER, ROWW>(p, rows, st);
     if (p.n_cols % 8 != 0 || p.kc % 8 != 0) return OM_ERR_SHAPE;
     if (p.kc % 64 != 0) return launch_rows<128, 128, AKIND, BKIND, EPI, GATHER, ROWW, true>(p, rows, st);
+    // Few rows per expert (fewer than 256 on average): the launch streams weights that are used once, and the
+    // kernels that keep two steps of them in flight are 4-10 % faster; with more rows the direct-load kernels
+    // are (4-9 % at 2000 rows per expert), so each regime gets its own.
+    if (rows < static_cast<int64_t>(p.n_experts) * 256)
+        return launch_rows<128, 128, AKIND, BKIND, EPI, GATHER, ROWW, false, true>(p, rows, st);
     return launch_rows<128, 128, AKIND, BKIND, EPI, GATHER, ROWW>(p, rows, st);
 }
 
