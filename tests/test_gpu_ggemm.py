@@ -397,3 +397,41 @@ def test_operands_beyond_2_31_elements(cuda):
         yr.backward(dy[s0:s1].float().cpu())
         for name, w, r in zip(("dwg", "dwu", "dwd"), ws, p):
             assert_bf16_parity(w.grad[e], r.grad, *MLP_BARS["grad"], tag=f"beyond2^31 expert {e} {name}")
+
+
+@pytest.mark.parametrize("N,K", [(320, 192), (192, 2048), (1000, 328)])
+def test_few_rows_kernels_give_the_bits_of_the_direct_load_kernels(cuda, N, K):
+    """Experts with few rows run kernels that stage their operands through registers (the weights two
+    contraction steps ahead); they are meant to change when data arrives in LDS, not what is summed.
+    The same light experts are computed twice through the C ABI: alone (fewer than 256 rows per expert
+    on average: the register-staged kernels), and followed by one heavy expert that lifts the average
+    above 256 rows (the direct-load kernels; sizes that keep both launches on the 128x128 tile).  The
+    light experts' rows must agree bit for bit, forward and input gradient."""
+    from optimus import _native as n
+    from util import bits
+    g = torch.Generator().manual_seed(N + K)
+    G = 12
+    light = torch.randint(0, 90, (G,), generator=g)
+    light[3] = 0
+    rows_light = int(light.sum())
+    heavy = (G + 1) * 256 + 64 - rows_light          # lifts the mean above 256 rows per expert
+    cum_a = torch.zeros(G + 1, dtype=torch.int32); cum_a[1:] = torch.cumsum(light, 0)
+    cum_b = torch.cat([cum_a, torch.tensor([rows_light + heavy], dtype=torch.int32)])
+    rows_b = rows_light + heavy
+    x = torch.randn(rows_b, K, generator=g).to(torch.bfloat16).to(cuda)
+    dout = torch.randn(rows_b, N, generator=g).to(torch.bfloat16).to(cuda)
+    w = (torch.randn(G + 1, N, K, generator=g) * 0.05).to(torch.bfloat16).to(cuda)
+    P = n.ptr
+    res = []
+    for cum, rows, experts in ((cum_a, rows_light, G), (cum_b, rows_b, G + 1)):
+        cum = cum.to(cuda)
+        out = torch.zeros(rows_b, N, dtype=torch.bfloat16, device=cuda)
+        dx = torch.zeros(rows_b, K, dtype=torch.bfloat16, device=cuda)
+        n.check(n.lib().om_grouped_gemm_fwd(P(x), P(w), P(out), P(cum), rows, experts, N, K, 0, n.stream()), "fwd")
+        n.check(n.lib().om_grouped_gemm_dgrad(P(dout), P(w), P(dx), P(cum), rows, experts, N, K, 0, n.stream()), "dgrad")
+        torch.cuda.synchronize()
+        res.append((out[:rows_light], dx[:rows_light]))
+    assert rows_light < G * 256 and rows_b >= (G + 1) * 256
+    assert float(res[0][0].float().abs().max()) > 0
+    assert (bits(res[0][0]) == bits(res[1][0])).all()
+    assert (bits(res[0][1]) == bits(res[1][1])).all()
